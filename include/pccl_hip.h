@@ -1,0 +1,229 @@
+/*
+ * pccl_hip.h -- C ABI of libpccl_hip.so: the per-GPU reduction and placement
+ * compute of PCCL's reduce_scatter / all_gather, written for gfx950 (MI355X).
+ *
+ * The library replaces the torch/pybind11 extension module that the reference
+ * builds at run time (pccl/build_kernels.py:102-105 compiles pccl/src/pccl.cpp,
+ * all_gather.cpp, reduce_scatter.cpp and common.cu into a module named "pccl").
+ * It is torch-free: every argument is a plain pointer, size or enum, so it can
+ * be bound from ctypes, cffi, pybind11 or C.
+ *
+ * Model. P "virtual ranks" live on ONE GPU: rank r's send and receive buffers
+ * are ordinary device allocations in that GPU's HBM, and the MPI_Sendrecv the
+ * reference issues between two device kernels (pccl/src/reduce_scatter.cpp:67-69,
+ * :140-142; pccl/src/all_gather.cpp:61-63) becomes a direct read of the
+ * partner's buffer by the kernel of the next step.  No inter-GPU collective is
+ * ever issued.
+ *
+ * Conventions
+ *  - Every entry point returns 0 on success and a negative PCCL_HIP_E* code on
+ *    failure; pccl_hip_last_error() then holds a message for the calling
+ *    thread.  Nothing here prints or terminates the process (the reference's
+ *    CUDA_CHECK calls exit(1): pccl/include/common.h:8-15).
+ *  - Pointer tables (void* const*) are HOST arrays of DEVICE pointers; they are
+ *    consumed before the call returns (copied into kernel arguments).
+ *  - The library never allocates, frees or retains device memory: the caller
+ *    passes inputs, outputs and workspaces (the reference shim allocates them
+ *    as torch tensors for the same reason: pccl/src/pccl.cpp:54-59,71-73).
+ *  - Work is only enqueued on `stream` (a hipStream_t; NULL = the default
+ *    stream).  No call synchronises the host.
+ *  - Sizes are size_t elements unless a name says bytes.  The reference uses
+ *    `int` for both (pccl/include/reduce_scatter.h:8,15, all_gather.h:8), so it
+ *    cannot address a 2 GiB buffer; this ABI can.
+ *  - Buffers passed to one call must not overlap except where a function
+ *    documents in-place use.
+ */
+#ifndef PCCL_HIP_H
+#define PCCL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PCCL_HIP_ABI_VERSION 1
+
+/* Largest number of ranks / shards / segments one call accepts. */
+#define PCCL_HIP_MAX_RANKS 64
+
+/* Element types.  bf16 sums are computed as RNE_bf16(float(a) + float(b)) at
+ * every hop, which is what torch.add does on bfloat16 tensors in the
+ * reference's Python algorithms (pccl/reduce_scatter.py:24,83,95,106,158). */
+enum pccl_hip_dtype {
+  PCCL_HIP_F32 = 0,
+  PCCL_HIP_BF16 = 1
+};
+
+/* Summation orders for the fused reduce (bit-exact replay of a schedule). */
+enum pccl_hip_order {
+  /* Left fold over ranks first, first+1, ... (mod k), i.e. the order in which
+   * the ring of pccl/src/reduce_scatter.cpp:127-146 accumulates block j when
+   * first = (j + 1) mod P. */
+  PCCL_HIP_ORDER_RING = 0,
+  /* XOR butterfly of recursive halving (pccl/src/reduce_scatter.cpp:50-89):
+   * v[m] = shard[first ^ m]; for h = k/2 .. 1: v[m] += v[m + h], m < h. */
+  PCCL_HIP_ORDER_HALVING = 1
+};
+
+/* How a whole collective is executed on the virtual ranks. */
+enum pccl_hip_mode {
+  /* One batched launch per step of the reference schedule; the input->work
+   * copy and the final copy-out are folded into the first and last step. */
+  PCCL_HIP_MODE_STEPS = 0,
+  /* One launch for the whole collective (k-way reduce / direct placement),
+   * reproducing the same summation order. */
+  PCCL_HIP_MODE_FUSED = 1,
+  /* The reference's memory operations one for one: copy input to the work
+   * buffer, add in place per step, copy the result block out
+   * (pccl/src/reduce_scatter.cpp:32-36,92-96,119-123,148-152). */
+  PCCL_HIP_MODE_FAITHFUL = 2
+};
+
+enum pccl_hip_status {
+  PCCL_HIP_OK = 0,
+  PCCL_HIP_EINVAL = -1,   /* bad argument (message says which) */
+  PCCL_HIP_ELAUNCH = -2,  /* the HIP runtime refused a launch */
+  PCCL_HIP_ENODEV = -3    /* no usable gfx950 device */
+};
+
+/* ABI version of the loaded library (== PCCL_HIP_ABI_VERSION). */
+int pccl_hip_version(void);
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char* pccl_hip_last_error(void);
+
+/* Size in bytes of one element of `dtype`, 0 if unknown. */
+size_t pccl_hip_dtype_size(int dtype);
+
+/* ---- a1: the accumulate kernel ------------------------------------------
+ * dst[i] = dst[i] + src[i], i < n.  Replaces vectorAdd / vectorAddKernel
+ * (pccl/src/common.cu:5-19; float only there).  Same result bits as the
+ * reference for fp32 (one IEEE add per element). */
+int pccl_hip_accumulate(void* dst, const void* src, size_t n, int dtype,
+                        void* stream);
+
+/* dst[i] = a[i] + b[i].  dst may alias a or b exactly (in-place), but must
+ * not partially overlap either.  This three-address form is what lets a
+ * schedule skip the reference's input->work copy. */
+int pccl_hip_add(void* dst, const void* a, const void* b, size_t n, int dtype,
+                 void* stream);
+
+/* `count` independent adds of n elements each in ONE launch:
+ * dst[s][i] = a[s][i] + b[s][i].  One ring step or halving round over all
+ * virtual ranks is one such call.  Segments must be pairwise hazard-free
+ * (no segment writes what another reads or writes). count <= PCCL_HIP_MAX_RANKS. */
+int pccl_hip_add_batched(void* const* dst, const void* const* a,
+                         const void* const* b, int count, size_t n, int dtype,
+                         void* stream);
+
+/* ---- a3: strided-half pairwise kernel (one recursive-halving round) -------
+ * bufs[r] is rank r's work buffer of P*B elements.  Round `round`
+ * (0 <= round < log2 P), group = P >> round, half = group/2 blocks,
+ * count = half*B, start(r) = (r / group) * group * B:
+ *   lower rank k (k % group <  half), partner p = k + half:
+ *       bufs[k][start : start+count]          += bufs[p][start : start+count]
+ *   upper rank p:
+ *       bufs[p][start+count : start+2*count]  += bufs[k][start+count : start+2*count]
+ * exactly the two branches of pccl/src/reduce_scatter.cpp:58-88 with the
+ * received half read from the partner's buffer.  All P ranks in one launch.
+ * If `src` is non-NULL the operands are read from src[] instead of bufs[]
+ * (first round straight from the inputs); if `outs` is non-NULL the sums of
+ * the LAST round (count == B) are written to outs[r][0:B] instead. */
+int pccl_hip_rh_round(void* const* bufs, const void* const* src,
+                      void* const* outs, int P, size_t B, int round, int dtype,
+                      void* stream);
+
+/* ---- fused one-pass k-way reduce -----------------------------------------
+ * out[i] = sum over the k shards of shard[.][i], i < n, added in `order`
+ * starting from shard `first`.  With per_hop_round != 0 a bf16 partial sum is
+ * rounded to bf16 after every add (bit-exact to k-1 calls of
+ * pccl_hip_accumulate); with 0 the partial sum stays in fp32 and is rounded
+ * once.  For PCCL_HIP_F32 the flag has no effect.  2 <= k <= PCCL_HIP_MAX_RANKS;
+ * PCCL_HIP_ORDER_HALVING needs k to be a power of two.  out must not overlap
+ * any shard. */
+int pccl_hip_reduce_kway(void* out, const void* const* shards, int k, size_t n,
+                         int dtype, int order, int first, int per_hop_round,
+                         void* stream);
+
+/* ---- placement copies ---------------------------------------------------
+ * `count` independent byte copies in one launch: dst[s][0:nbytes[s]] =
+ * src[s][0:nbytes[s]].  Any alignment and any size (0 allowed); 16-byte
+ * aligned segments take the 128-bit path.  count <= PCCL_HIP_MAX_RANKS.
+ * Replaces the cudaMemcpyAsync placement copies of pccl/src/all_gather.cpp:31-35
+ * and pccl/src/reduce_scatter.cpp:32-36,92-96,119-123,148-152. */
+int pccl_hip_copy_batched(void* const* dst, const void* const* src,
+                          const size_t* nbytes, int count, void* stream);
+
+/* out[dst_off[k] : dst_off[k] + nbytes[k]] = shard[k][0 : nbytes[k]] for
+ * k < P: materialise one rank's all_gather output from the P shards in one
+ * launch.  Uneven shards are expressed by nbytes[]/dst_off[] (bytes); gaps
+ * between shards (padding) are left untouched. */
+int pccl_hip_gather_place(void* out, const void* const* shards,
+                          const size_t* nbytes, const size_t* dst_off, int P,
+                          void* stream);
+
+/* dst viewed as [cols][rows][m] = src viewed as [rows][cols][m], m in bytes:
+ * the block transpose that reduce_scatter_2D applies before the inner
+ * collective (pccl/reduce_scatter.py:226, rows = inter, cols = intra) and
+ * all_gather_2D applies after it (pccl/all_gather.py:158-159, rows = intra,
+ * cols = inter).  dst must not overlap src. */
+int pccl_hip_block_transpose(void* dst, const void* src, size_t rows,
+                             size_t cols, size_t m_bytes, void* stream);
+
+/* ---- whole collectives on virtual ranks -----------------------------------
+ * reduce_scatter over P virtual ranks.  Replaces reduce_scatter_mpi
+ * (pccl/src/pccl.cpp:11-85) and the two algorithms it dispatches to
+ * (pccl/src/reduce_scatter.cpp:16-99 "recursive", :101-155 "ring").
+ *   inputs[r]  : rank r's input, P*B elements (read only)
+ *   outputs[r] : rank r's output, B elements = sum_k inputs[k][r*B:(r+1)*B]
+ *   work[r]    : rank r's workspace, P*B elements; may be NULL as a whole
+ *                for PCCL_HIP_MODE_FUSED and for P <= 2
+ *   algorithm  : "ring" or "recursive" (recursive needs P a power of two);
+ *                any other string is an error, as at pccl.cpp:83.
+ * The summation order of each output block is that of the named algorithm in
+ * every mode.  1 <= P <= PCCL_HIP_MAX_RANKS. */
+int pccl_hip_reduce_scatter_virtual(void* const* outputs,
+                                    const void* const* inputs,
+                                    void* const* work, int P, size_t B,
+                                    int dtype, const char* algorithm, int mode,
+                                    void* stream);
+
+/* all_gather over P virtual ranks, in bytes.  Replaces all_gather_mpi
+ * (pccl/src/pccl.cpp:87-142) and recursiveDoublingAllGatherGPU
+ * (pccl/src/all_gather.cpp:15-69).
+ *   inputs[r]  : rank r's shard, block_bytes bytes
+ *   outputs[r] : rank r's output, P*block_bytes bytes = concatenation of the
+ *                shards in rank order
+ *   algorithm  : "recursive" (doubling, P a power of two) or "ring"
+ *                (the ring schedule the reference leaves to MPI_Allgather,
+ *                pccl/all_gather.py:124-128).
+ * PCCL_HIP_MODE_STEPS replays one batched copy per step;
+ * PCCL_HIP_MODE_FUSED places every shard directly; FAITHFUL == STEPS. */
+int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs,
+                                int P, size_t block_bytes,
+                                const char* algorithm, int mode, void* stream);
+
+/* Uneven all_gather: shard k has nbytes[k] bytes and lands at byte offset
+ * dst_off[k] of every output (the caller chooses offsets, e.g. each shard
+ * padded to a multiple of 256 bytes).  One launch places all P*P segments.
+ * Not a reference feature (it requires equal shards, pccl/src/pccl.cpp:111-116). */
+int pccl_hip_all_gather_uneven_virtual(void* const* outputs,
+                                       const void* const* inputs,
+                                       const size_t* nbytes,
+                                       const size_t* dst_off, int P,
+                                       void* stream);
+
+/* ---- launch tuning (for measurement) ------------------------------------
+ * key: "grid_cap" (max workgroups per launch, 0 = one tile per workgroup),
+ *      "unroll"   (128-bit vectors per thread per operand: 1, 2, 4 or 8),
+ *      "nt_load" / "nt_store" (0/1: non-temporal global loads / stores).
+ * Returns 0, or PCCL_HIP_EINVAL for an unknown key or value.  Process-wide. */
+int pccl_hip_set_tuning(const char* key, long value);
+long pccl_hip_get_tuning(const char* key);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PCCL_HIP_H */

@@ -1,0 +1,613 @@
+// libpccl_hip.so -- reduction and placement kernels of PCCL's collectives for
+// gfx950 (MI355X), behind the C ABI declared in include/pccl_hip.h.
+//
+// Everything here is HBM-bandwidth bound (one add per 6-12 bytes, or a pure
+// copy), so the kernels are organised around memory traffic only:
+//   * every global access is a 128-bit load/store, consecutive lanes touch
+//     consecutive 16-byte vectors (one wave instruction = 1 KiB contiguous);
+//   * each thread issues all loads of its tile before the first use, so a
+//     workgroup of 256 threads keeps 2*U*4 KiB of reads in flight (U = vectors
+//     per thread and operand);
+//   * a whole step of a schedule (all virtual ranks) is ONE launch: the
+//     per-segment pointers travel in the kernel arguments, so nothing is
+//     allocated or copied to the device to describe the step;
+//   * workgroups walk the segments tile by tile in address order.
+// No MFMA: there is no contraction anywhere on this path.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+
+#include "pccl_hip.h"
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// errors and tuning
+// ---------------------------------------------------------------------------
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof g_err, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int launch_status(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    return fail(PCCL_HIP_ELAUNCH, "%s: launch failed: %s", what, hipGetErrorString(e));
+  return PCCL_HIP_OK;
+}
+
+std::atomic<long> g_grid_cap{0};
+std::atomic<long> g_unroll{4};
+std::atomic<long> g_nt_load{0};
+std::atomic<long> g_nt_store{0};
+
+}  // namespace
+
+#include "pccl_kernels.h"
+
+namespace {
+
+using namespace pccl_kernels;
+
+// ---------------------------------------------------------------------------
+// host side: launch geometry and dispatch over the tuning parameters
+// ---------------------------------------------------------------------------
+unsigned grid_for(size_t total_tiles) {
+  long cap = g_grid_cap.load(std::memory_order_relaxed);
+  size_t g = total_tiles;
+  if (cap > 0 && g > (size_t)cap) g = (size_t)cap;
+  if (g > kMaxGrid) g = kMaxGrid;
+  if (g == 0) g = 1;
+  return (unsigned)g;
+}
+
+size_t tiles_for(size_t nbytes, int unroll) {
+  // one extra vector covers the shift of the body behind an unaligned head
+  size_t nvec = nbytes / 16 + 2;
+  size_t per = (size_t)kThreads * (size_t)unroll;
+  return (nvec + per - 1) / per;
+}
+
+struct Tune {
+  int unroll;
+  bool ntl, nts;
+};
+
+Tune current_tune() {
+  Tune t;
+  t.unroll = (int)g_unroll.load(std::memory_order_relaxed);
+  t.ntl = g_nt_load.load(std::memory_order_relaxed) != 0;
+  t.nts = g_nt_store.load(std::memory_order_relaxed) != 0;
+  return t;
+}
+
+// Calls f.template operator()<U, NTL, NTS>() for the current tuning.
+template <class F>
+void with_tuning(const Tune& t, F&& f) {
+#define PCCL_CASE(UV)                                                 \
+  case UV:                                                            \
+    if (t.ntl) {                                                      \
+      if (t.nts) f.template operator()<UV, true, true>();             \
+      else f.template operator()<UV, true, false>();                  \
+    } else {                                                          \
+      if (t.nts) f.template operator()<UV, false, true>();            \
+      else f.template operator()<UV, false, false>();                 \
+    }                                                                 \
+    break;
+  switch (t.unroll) {
+    PCCL_CASE(1)
+    PCCL_CASE(2)
+    PCCL_CASE(8)
+    default:
+    PCCL_CASE(4)
+  }
+#undef PCCL_CASE
+}
+
+size_t esize_of(int dtype) {
+  return dtype == PCCL_HIP_F32 ? 4 : dtype == PCCL_HIP_BF16 ? 2 : 0;
+}
+
+struct AddLaunch {
+  const AddSegs* segs;
+  int count, dtype;
+  size_t n, tiles;
+  hipStream_t stream;
+  template <int U, bool NTL, bool NTS>
+  void operator()() const {
+    unsigned grid = grid_for((size_t)count * tiles);
+    if (dtype == PCCL_HIP_F32)
+      hipLaunchKernelGGL((k_add_segs<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, n, tiles);
+    else
+      hipLaunchKernelGGL((k_add_segs<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, n, tiles);
+  }
+};
+
+int launch_add(const AddSegs& segs, int count, size_t n, int dtype, hipStream_t stream,
+               const char* what) {
+  if (n == 0 || count == 0) return PCCL_HIP_OK;
+  Tune t = current_tune();
+  AddLaunch l{&segs, count, dtype, n, tiles_for(n * esize_of(dtype), t.unroll), stream};
+  with_tuning(t, l);
+  return launch_status(what);
+}
+
+struct CopyLaunch {
+  const CopySegs* segs;
+  int count;
+  size_t tiles;
+  hipStream_t stream;
+  template <int U, bool NTL, bool NTS>
+  void operator()() const {
+    unsigned grid = grid_for((size_t)count * tiles);
+    hipLaunchKernelGGL((k_copy_segs<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, tiles);
+  }
+};
+
+int launch_copy(const CopySegs& segs, int count, hipStream_t stream, const char* what) {
+  size_t longest = 0;
+  for (int s = 0; s < count; ++s) longest = segs.nbytes[s] > longest ? segs.nbytes[s] : longest;
+  if (longest == 0 || count == 0) return PCCL_HIP_OK;
+  Tune t = current_tune();
+  CopyLaunch l{&segs, count, tiles_for(longest, t.unroll), stream};
+  with_tuning(t, l);
+  return launch_status(what);
+}
+
+struct RhLaunch {
+  const RhArgs* args;
+  int P, round, dtype, from_src, to_outs;
+  size_t B, tiles;
+  hipStream_t stream;
+  template <int U, bool NTL, bool NTS>
+  void operator()() const {
+    unsigned grid = grid_for((size_t)P * tiles);
+    if (dtype == PCCL_HIP_F32)
+      hipLaunchKernelGGL((k_rh_round<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *args, P, B, round, from_src,
+                                                                    to_outs, tiles);
+    else
+      hipLaunchKernelGGL((k_rh_round<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *args, P, B, round, from_src,
+                                                                     to_outs, tiles);
+  }
+};
+
+struct GatherLaunch {
+  const GatherArgs* args;
+  int P, nout;
+  size_t tiles;
+  hipStream_t stream;
+  template <int U, bool NTL, bool NTS>
+  void operator()() const {
+    unsigned grid = grid_for((size_t)P * tiles);
+    hipLaunchKernelGGL((k_gather_multicast<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *args, P, nout, tiles);
+  }
+};
+
+struct TransposeLaunch {
+  uint8_t* dst;
+  const uint8_t* src;
+  size_t rows, cols, m, tiles;
+  hipStream_t stream;
+  template <int U, bool NTL, bool NTS>
+  void operator()() const {
+    unsigned grid = grid_for(rows * cols * tiles);
+    hipLaunchKernelGGL((k_block_transpose<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, dst, src, rows, cols, m, tiles);
+  }
+};
+
+// The fused reduce keeps more live registers per vector, so it uses at most
+// two vectors per thread.
+struct KwayLaunch {
+  const KwayArgs* args;
+  int k, nout, dtype, order, first0, per_hop;
+  size_t stride, n;
+  hipStream_t stream;
+
+  template <class Acc, int U, bool NTL, bool NTS>
+  void run() const {
+    size_t tiles = tiles_for(n * sizeof(typename Acc::op::elem), U);
+    unsigned grid = grid_for((size_t)nout * tiles);
+#define PCCL_KWAY(KV) \
+  hipLaunchKernelGGL((k_reduce_kway<Acc, KV, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *args, k, nout, stride, n, first0, tiles)
+    if (order == PCCL_HIP_ORDER_RING) { PCCL_KWAY(0); return; }
+    switch (k) {
+      case 2: PCCL_KWAY(2); break;
+      case 4: PCCL_KWAY(4); break;
+      case 8: PCCL_KWAY(8); break;
+      case 16: PCCL_KWAY(16); break;
+      case 32: PCCL_KWAY(32); break;
+      default: PCCL_KWAY(64); break;
+    }
+#undef PCCL_KWAY
+  }
+
+  template <int U, bool NTL, bool NTS>
+  void operator()() const {
+    constexpr int UK = U > 2 ? 2 : U;
+    if (dtype == PCCL_HIP_F32) run<AccF32, UK, NTL, NTS>();
+    else if (per_hop) run<AccBF16<true>, UK, NTL, NTS>();
+    else run<AccBF16<false>, UK, NTL, NTS>();
+  }
+};
+
+int launch_kway(const KwayArgs& args, int k, int nout, size_t stride, size_t n, int dtype, int order,
+                int first0, int per_hop, hipStream_t stream, const char* what) {
+  if (n == 0 || nout == 0) return PCCL_HIP_OK;
+  KwayLaunch l{&args, k, nout, dtype, order, first0, per_hop, stride, n, stream};
+  with_tuning(current_tune(), l);
+  return launch_status(what);
+}
+
+bool pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+
+int check_table(const void* const* tab, int count, const char* what, const char* name) {
+  if (!tab) return fail(PCCL_HIP_EINVAL, "%s: %s is NULL", what, name);
+  for (int i = 0; i < count; ++i)
+    if (!tab[i]) return fail(PCCL_HIP_EINVAL, "%s: %s[%d] is NULL", what, name, i);
+  return PCCL_HIP_OK;
+}
+
+int check_dtype(int dtype, const char* what) {
+  if (esize_of(dtype) == 0)
+    return fail(PCCL_HIP_EINVAL, "%s: unknown dtype %d (0 = float32, 1 = bfloat16)", what, dtype);
+  return PCCL_HIP_OK;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------
+extern "C" {
+
+int pccl_hip_version(void) { return PCCL_HIP_ABI_VERSION; }
+
+const char* pccl_hip_last_error(void) { return g_err; }
+
+size_t pccl_hip_dtype_size(int dtype) { return esize_of(dtype); }
+
+int pccl_hip_set_tuning(const char* key, long value) {
+  if (!key) return fail(PCCL_HIP_EINVAL, "set_tuning: key is NULL");
+  if (!strcmp(key, "grid_cap")) {
+    if (value < 0) return fail(PCCL_HIP_EINVAL, "set_tuning: grid_cap must be >= 0");
+    g_grid_cap = value;
+  } else if (!strcmp(key, "unroll")) {
+    if (value != 1 && value != 2 && value != 4 && value != 8)
+      return fail(PCCL_HIP_EINVAL, "set_tuning: unroll must be 1, 2, 4 or 8");
+    g_unroll = value;
+  } else if (!strcmp(key, "nt_load")) {
+    g_nt_load = value != 0;
+  } else if (!strcmp(key, "nt_store")) {
+    g_nt_store = value != 0;
+  } else {
+    return fail(PCCL_HIP_EINVAL, "set_tuning: unknown key '%s'", key);
+  }
+  return PCCL_HIP_OK;
+}
+
+long pccl_hip_get_tuning(const char* key) {
+  if (!key) return -1;
+  if (!strcmp(key, "grid_cap")) return g_grid_cap;
+  if (!strcmp(key, "unroll")) return g_unroll;
+  if (!strcmp(key, "nt_load")) return g_nt_load;
+  if (!strcmp(key, "nt_store")) return g_nt_store;
+  return -1;
+}
+
+int pccl_hip_add(void* dst, const void* a, const void* b, size_t n, int dtype, void* stream) {
+  const char* what = "pccl_hip_add";
+  if (int rc = check_dtype(dtype, what)) return rc;
+  if (n == 0) return PCCL_HIP_OK;
+  if (!dst || !a || !b) return fail(PCCL_HIP_EINVAL, "%s: NULL operand", what);
+  AddSegs segs;
+  segs.dst[0] = dst; segs.a[0] = a; segs.b[0] = b;
+  return launch_add(segs, 1, n, dtype, (hipStream_t)stream, what);
+}
+
+int pccl_hip_accumulate(void* dst, const void* src, size_t n, int dtype, void* stream) {
+  const char* what = "pccl_hip_accumulate";
+  if (int rc = check_dtype(dtype, what)) return rc;
+  if (n == 0) return PCCL_HIP_OK;
+  if (!dst || !src) return fail(PCCL_HIP_EINVAL, "%s: NULL operand", what);
+  AddSegs segs;
+  segs.dst[0] = dst; segs.a[0] = dst; segs.b[0] = src;
+  return launch_add(segs, 1, n, dtype, (hipStream_t)stream, what);
+}
+
+int pccl_hip_add_batched(void* const* dst, const void* const* a, const void* const* b, int count,
+                         size_t n, int dtype, void* stream) {
+  const char* what = "pccl_hip_add_batched";
+  if (int rc = check_dtype(dtype, what)) return rc;
+  if (count < 0 || count > kMaxSeg)
+    return fail(PCCL_HIP_EINVAL, "%s: count %d outside [0, %d]", what, count, kMaxSeg);
+  if (count == 0 || n == 0) return PCCL_HIP_OK;
+  if (int rc = check_table((const void* const*)dst, count, what, "dst")) return rc;
+  if (int rc = check_table(a, count, what, "a")) return rc;
+  if (int rc = check_table(b, count, what, "b")) return rc;
+  AddSegs segs;
+  for (int s = 0; s < count; ++s) { segs.dst[s] = dst[s]; segs.a[s] = a[s]; segs.b[s] = b[s]; }
+  return launch_add(segs, count, n, dtype, (hipStream_t)stream, what);
+}
+
+int pccl_hip_rh_round(void* const* bufs, const void* const* src, void* const* outs, int P, size_t B,
+                      int round, int dtype, void* stream) {
+  const char* what = "pccl_hip_rh_round";
+  if (int rc = check_dtype(dtype, what)) return rc;
+  if (P < 2 || P > kMaxSeg || !pow2(P))
+    return fail(PCCL_HIP_EINVAL, "%s: P = %d must be a power of two in [2, %d]", what, P, kMaxSeg);
+  int rounds = 0;
+  while ((1 << rounds) < P) ++rounds;
+  if (round < 0 || round >= rounds)
+    return fail(PCCL_HIP_EINVAL, "%s: round %d outside [0, %d)", what, round, rounds);
+  const bool last = round == rounds - 1;
+  const bool to_outs = outs != nullptr && last;
+  // the work buffers are needed unless this round reads the inputs and writes the outputs
+  const bool need_bufs = !(src != nullptr && to_outs);
+  if (need_bufs) if (int rc = check_table((const void* const*)bufs, P, what, "bufs")) return rc;
+  if (src) if (int rc = check_table(src, P, what, "src")) return rc;
+  if (to_outs) if (int rc = check_table((const void* const*)outs, P, what, "outs")) return rc;
+  if (B == 0) return PCCL_HIP_OK;
+  RhArgs args;
+  for (int r = 0; r < P; ++r) {
+    args.bufs[r] = need_bufs ? bufs[r] : nullptr;
+    args.src[r] = src ? src[r] : nullptr;
+    args.outs[r] = to_outs ? outs[r] : nullptr;
+  }
+  const size_t count = (size_t)((P >> round) / 2) * B;
+  Tune t = current_tune();
+  RhLaunch l{&args, P, round, dtype, src ? 1 : 0, to_outs ? 1 : 0, B,
+             tiles_for(count * esize_of(dtype), t.unroll), (hipStream_t)stream};
+  with_tuning(t, l);
+  return launch_status(what);
+}
+
+int pccl_hip_reduce_kway(void* out, const void* const* shards, int k, size_t n, int dtype,
+                         int order, int first, int per_hop_round, void* stream) {
+  const char* what = "pccl_hip_reduce_kway";
+  if (int rc = check_dtype(dtype, what)) return rc;
+  if (k < 2 || k > kMaxSeg) return fail(PCCL_HIP_EINVAL, "%s: k = %d outside [2, %d]", what, k, kMaxSeg);
+  if (order != PCCL_HIP_ORDER_RING && order != PCCL_HIP_ORDER_HALVING)
+    return fail(PCCL_HIP_EINVAL, "%s: unknown order %d", what, order);
+  if (order == PCCL_HIP_ORDER_HALVING && !pow2(k))
+    return fail(PCCL_HIP_EINVAL, "%s: halving order needs k = %d to be a power of two", what, k);
+  if (first < 0 || first >= k) return fail(PCCL_HIP_EINVAL, "%s: first = %d outside [0, %d)", what, first, k);
+  if (n == 0) return PCCL_HIP_OK;
+  if (!out) return fail(PCCL_HIP_EINVAL, "%s: out is NULL", what);
+  if (int rc = check_table(shards, k, what, "shards")) return rc;
+  KwayArgs args;
+  for (int q = 0; q < k; ++q) args.shard[q] = shards[q];
+  args.out[0] = out;
+  return launch_kway(args, k, 1, 0, n, dtype, order, first, per_hop_round, (hipStream_t)stream, what);
+}
+
+int pccl_hip_copy_batched(void* const* dst, const void* const* src, const size_t* nbytes, int count,
+                          void* stream) {
+  const char* what = "pccl_hip_copy_batched";
+  if (count < 0 || count > kMaxSeg)
+    return fail(PCCL_HIP_EINVAL, "%s: count %d outside [0, %d]", what, count, kMaxSeg);
+  if (count == 0) return PCCL_HIP_OK;
+  if (!nbytes) return fail(PCCL_HIP_EINVAL, "%s: nbytes is NULL", what);
+  if (!dst || !src) return fail(PCCL_HIP_EINVAL, "%s: NULL pointer table", what);
+  CopySegs segs;
+  for (int s = 0; s < count; ++s) {
+    if (nbytes[s] && (!dst[s] || !src[s]))
+      return fail(PCCL_HIP_EINVAL, "%s: segment %d has a NULL pointer", what, s);
+    segs.dst[s] = dst[s]; segs.src[s] = src[s]; segs.nbytes[s] = nbytes[s];
+  }
+  return launch_copy(segs, count, (hipStream_t)stream, what);
+}
+
+int pccl_hip_gather_place(void* out, const void* const* shards, const size_t* nbytes,
+                          const size_t* dst_off, int P, void* stream) {
+  const char* what = "pccl_hip_gather_place";
+  if (P < 1 || P > kMaxSeg) return fail(PCCL_HIP_EINVAL, "%s: P = %d outside [1, %d]", what, P, kMaxSeg);
+  if (!out || !shards || !nbytes || !dst_off) return fail(PCCL_HIP_EINVAL, "%s: NULL argument", what);
+  CopySegs segs;
+  for (int k = 0; k < P; ++k) {
+    if (nbytes[k] && !shards[k]) return fail(PCCL_HIP_EINVAL, "%s: shards[%d] is NULL", what, k);
+    segs.dst[k] = (uint8_t*)out + dst_off[k]; segs.src[k] = shards[k]; segs.nbytes[k] = nbytes[k];
+  }
+  return launch_copy(segs, P, (hipStream_t)stream, what);
+}
+
+int pccl_hip_block_transpose(void* dst, const void* src, size_t rows, size_t cols, size_t m_bytes,
+                             void* stream) {
+  const char* what = "pccl_hip_block_transpose";
+  if (rows == 0 || cols == 0 || m_bytes == 0) return PCCL_HIP_OK;
+  if (!dst || !src) return fail(PCCL_HIP_EINVAL, "%s: NULL operand", what);
+  Tune t = current_tune();
+  TransposeLaunch l{(uint8_t*)dst, (const uint8_t*)src, rows, cols, m_bytes,
+                    tiles_for(m_bytes, t.unroll), (hipStream_t)stream};
+  with_tuning(t, l);
+  return launch_status(what);
+}
+
+int pccl_hip_all_gather_uneven_virtual(void* const* outputs, const void* const* inputs,
+                                       const size_t* nbytes, const size_t* dst_off, int P,
+                                       void* stream) {
+  const char* what = "pccl_hip_all_gather_uneven_virtual";
+  if (P < 1 || P > kMaxSeg) return fail(PCCL_HIP_EINVAL, "%s: P = %d outside [1, %d]", what, P, kMaxSeg);
+  if (!nbytes || !dst_off) return fail(PCCL_HIP_EINVAL, "%s: NULL size table", what);
+  if (int rc = check_table((const void* const*)outputs, P, what, "outputs")) return rc;
+  if (!inputs) return fail(PCCL_HIP_EINVAL, "%s: inputs is NULL", what);
+  GatherArgs args;
+  size_t longest = 0;
+  for (int k = 0; k < P; ++k) {
+    if (nbytes[k] && !inputs[k]) return fail(PCCL_HIP_EINVAL, "%s: inputs[%d] is NULL", what, k);
+    args.outs[k] = outputs[k]; args.ins[k] = inputs[k];
+    args.nbytes[k] = nbytes[k]; args.dst_off[k] = dst_off[k];
+    longest = nbytes[k] > longest ? nbytes[k] : longest;
+  }
+  if (longest == 0) return PCCL_HIP_OK;
+  Tune t = current_tune();
+  GatherLaunch l{&args, P, P, tiles_for(longest, t.unroll), (hipStream_t)stream};
+  with_tuning(t, l);
+  return launch_status(what);
+}
+
+int pccl_hip_reduce_scatter_virtual(void* const* outputs, const void* const* inputs,
+                                    void* const* work, int P, size_t B, int dtype,
+                                    const char* algorithm, int mode, void* stream) {
+  const char* what = "pccl_hip_reduce_scatter_virtual";
+  if (int rc = check_dtype(dtype, what)) return rc;
+  if (!algorithm) return fail(PCCL_HIP_EINVAL, "%s: algorithm is NULL", what);
+  const bool ring = !strcmp(algorithm, "ring");
+  const bool rec = !strcmp(algorithm, "recursive");
+  if (!ring && !rec)
+    return fail(PCCL_HIP_EINVAL, "Unknown algorithm specified for reduce_scatter_mpi: %s", algorithm);
+  if (P < 1 || P > kMaxSeg) return fail(PCCL_HIP_EINVAL, "%s: P = %d outside [1, %d]", what, P, kMaxSeg);
+  if (rec && !pow2(P))
+    return fail(PCCL_HIP_EINVAL, "%s: recursive halving needs a power-of-two P, got %d", what, P);
+  if (mode != PCCL_HIP_MODE_STEPS && mode != PCCL_HIP_MODE_FUSED && mode != PCCL_HIP_MODE_FAITHFUL)
+    return fail(PCCL_HIP_EINVAL, "%s: unknown mode %d", what, mode);
+  if (int rc = check_table((const void* const*)outputs, P, what, "outputs")) return rc;
+  if (int rc = check_table(inputs, P, what, "inputs")) return rc;
+  const bool need_work = (mode == PCCL_HIP_MODE_FAITHFUL && P > 1) || (mode == PCCL_HIP_MODE_STEPS && P > 2);
+  if (need_work) if (int rc = check_table((const void* const*)work, P, what, "work")) return rc;
+  if (B == 0) return PCCL_HIP_OK;
+  hipStream_t st = (hipStream_t)stream;
+  const size_t es = esize_of(dtype);
+
+  if (P == 1) {  // zero steps: the output is the input block
+    CopySegs c;
+    c.dst[0] = outputs[0]; c.src[0] = inputs[0]; c.nbytes[0] = B * es;
+    return launch_copy(c, 1, st, what);
+  }
+
+  if (mode == PCCL_HIP_MODE_FUSED) {
+    KwayArgs args;
+    for (int r = 0; r < P; ++r) { args.shard[r] = inputs[r]; args.out[r] = outputs[r]; }
+    // ring: block j is folded from rank j+1 on; halving: the butterfly rooted at rank j
+    return launch_kway(args, P, P, B, B, dtype, ring ? PCCL_HIP_ORDER_RING : PCCL_HIP_ORDER_HALVING,
+                       ring ? 1 : 0, 1, st, what);
+  }
+
+  const bool faithful = mode == PCCL_HIP_MODE_FAITHFUL;
+  if (faithful) {  // buf <- input
+    CopySegs c;
+    for (int r = 0; r < P; ++r) { c.dst[r] = work[r]; c.src[r] = inputs[r]; c.nbytes[r] = (size_t)P * B * es; }
+    if (int rc = launch_copy(c, P, st, what)) return rc;
+  }
+
+  if (ring) {
+    for (int step = 0; step < P - 1; ++step) {
+      AddSegs segs;
+      const bool first = step == 0, last = step == P - 2;
+      for (int r = 0; r < P; ++r) {
+        const int recv_idx = ((r - step - 2) % P + P) % P;
+        const int source = (r - 1 + P) % P;
+        const size_t off = (size_t)recv_idx * B * es;
+        if (faithful) {
+          segs.dst[r] = (uint8_t*)work[r] + off;
+          segs.a[r] = segs.dst[r];
+          segs.b[r] = (const uint8_t*)work[source] + off;
+        } else {
+          // rank r's block recv_idx is still its input; the running sum of the
+          // left neighbour is its input at step 0 and its work buffer after
+          segs.a[r] = (const uint8_t*)inputs[r] + off;
+          segs.b[r] = first ? (const uint8_t*)inputs[source] + off : (const uint8_t*)work[source] + off;
+          segs.dst[r] = last ? outputs[r] : (void*)((uint8_t*)work[r] + off);
+        }
+      }
+      if (int rc = launch_add(segs, P, B, dtype, st, what)) return rc;
+    }
+    if (faithful) {
+      CopySegs c;
+      for (int r = 0; r < P; ++r) {
+        c.dst[r] = outputs[r]; c.src[r] = (const uint8_t*)work[r] + (size_t)r * B * es; c.nbytes[r] = B * es;
+      }
+      return launch_copy(c, P, st, what);
+    }
+    return PCCL_HIP_OK;
+  }
+
+  // recursive halving
+  int rounds = 0;
+  while ((1 << rounds) < P) ++rounds;
+  for (int round = 0; round < rounds; ++round) {
+    const bool from_inputs = !faithful && round == 0;
+    const bool to_outputs = !faithful && round == rounds - 1;
+    if (int rc = pccl_hip_rh_round(work, from_inputs ? inputs : nullptr, to_outputs ? outputs : nullptr, P,
+                                   B, round, dtype, stream))
+      return rc;
+  }
+  if (faithful) {
+    CopySegs c;
+    for (int r = 0; r < P; ++r) {
+      c.dst[r] = outputs[r]; c.src[r] = (const uint8_t*)work[r] + (size_t)r * B * es; c.nbytes[r] = B * es;
+    }
+    return launch_copy(c, P, st, what);
+  }
+  return PCCL_HIP_OK;
+}
+
+int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs, int P,
+                                size_t block_bytes, const char* algorithm, int mode, void* stream) {
+  const char* what = "pccl_hip_all_gather_virtual";
+  if (!algorithm) return fail(PCCL_HIP_EINVAL, "%s: algorithm is NULL", what);
+  const bool ring = !strcmp(algorithm, "ring");
+  const bool rec = !strcmp(algorithm, "recursive");
+  if (!ring && !rec)
+    return fail(PCCL_HIP_EINVAL, "Unknown algorithm specified for all_gather_mpi: %s", algorithm);
+  if (P < 1 || P > kMaxSeg) return fail(PCCL_HIP_EINVAL, "%s: P = %d outside [1, %d]", what, P, kMaxSeg);
+  if (rec && !pow2(P))
+    return fail(PCCL_HIP_EINVAL, "%s: recursive doubling needs a power-of-two P, got %d", what, P);
+  if (mode != PCCL_HIP_MODE_STEPS && mode != PCCL_HIP_MODE_FUSED && mode != PCCL_HIP_MODE_FAITHFUL)
+    return fail(PCCL_HIP_EINVAL, "%s: unknown mode %d", what, mode);
+  if (int rc = check_table((const void* const*)outputs, P, what, "outputs")) return rc;
+  if (int rc = check_table(inputs, P, what, "inputs")) return rc;
+  if (block_bytes == 0) return PCCL_HIP_OK;
+  hipStream_t st = (hipStream_t)stream;
+
+  if (mode == PCCL_HIP_MODE_FUSED) {
+    size_t nbytes[kMaxSeg], off[kMaxSeg];
+    for (int k = 0; k < P; ++k) { nbytes[k] = block_bytes; off[k] = (size_t)k * block_bytes; }
+    return pccl_hip_all_gather_uneven_virtual(outputs, inputs, nbytes, off, P, stream);
+  }
+
+  // out[r][r] <- in[r]   (pccl/src/all_gather.cpp:31-35)
+  CopySegs c;
+  for (int r = 0; r < P; ++r) {
+    c.dst[r] = (uint8_t*)outputs[r] + (size_t)r * block_bytes; c.src[r] = inputs[r]; c.nbytes[r] = block_bytes;
+  }
+  if (int rc = launch_copy(c, P, st, what)) return rc;
+
+  if (rec) {
+    for (int seg = 1; seg < P; seg *= 2) {
+      for (int r = 0; r < P; ++r) {
+        const int partner = r ^ seg;
+        const int group_start = (r / (2 * seg)) * (2 * seg);
+        const size_t recv_off = (size_t)(r < partner ? group_start + seg : group_start) * block_bytes;
+        // the partner's send offset equals this rank's receive offset
+        c.dst[r] = (uint8_t*)outputs[r] + recv_off;
+        c.src[r] = (const uint8_t*)outputs[partner] + recv_off;
+        c.nbytes[r] = (size_t)seg * block_bytes;
+      }
+      if (int rc = launch_copy(c, P, st, what)) return rc;
+    }
+    return PCCL_HIP_OK;
+  }
+
+  for (int step = 0; step < P - 1; ++step) {
+    for (int r = 0; r < P; ++r) {
+      const int j = ((r - step - 1) % P + P) % P;
+      const int source = (r - 1 + P) % P;
+      c.dst[r] = (uint8_t*)outputs[r] + (size_t)j * block_bytes;
+      c.src[r] = (const uint8_t*)outputs[source] + (size_t)j * block_bytes;
+      c.nbytes[r] = block_bytes;
+    }
+    if (int rc = launch_copy(c, P, st, what)) return rc;
+  }
+  return PCCL_HIP_OK;
+}
+
+}  // extern "C"

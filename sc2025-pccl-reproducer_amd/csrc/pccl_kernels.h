@@ -1,0 +1,522 @@
+// pccl_kernels.h -- device code of libpccl_hip.so: the gfx950 kernels for
+// PCCL's reduction and placement work.  Included by pccl_hip.hip only (and by
+// the host-side indexing check in tests/, which runs the same code thread by
+// thread on the CPU; the kernels use no LDS and no barriers, so that is exact).
+#ifndef PCCL_KERNELS_H
+#define PCCL_KERNELS_H
+
+#include <cstddef>
+#include <cstdint>
+
+#include "pccl_hip.h"
+
+namespace pccl_kernels {
+
+constexpr int kThreads = 256;              // 4 waves of 64 lanes
+constexpr int kMaxSeg = PCCL_HIP_MAX_RANKS;
+constexpr unsigned kMaxGrid = 0x7fffffffu;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// ---------------------------------------------------------------------------
+// device helpers
+// ---------------------------------------------------------------------------
+template <bool NT>
+__device__ __forceinline__ u32x4 ld16(const u32x4* p) {
+  if constexpr (NT) return __builtin_nontemporal_load(p);
+  else return *p;
+}
+
+template <bool NT>
+__device__ __forceinline__ void st16(u32x4* p, u32x4 v) {
+  if constexpr (NT) __builtin_nontemporal_store(v, p);
+  else *p = v;
+}
+
+// Round an fp32 value (given as bits) to bfloat16, ties to even; the result
+// stays in the upper 16 bits so that it is again a valid fp32 operand.
+// NaN becomes the canonical quiet NaN 0x7FC0, as on the host.
+__device__ __forceinline__ uint32_t bf16_round_hi(float s) {
+  uint32_t w = __float_as_uint(s);
+  uint32_t r = (w + 0x7fffu + ((w >> 16) & 1u)) & 0xffff0000u;
+  return (s != s) ? 0x7fc00000u : r;
+}
+
+struct OpF32 {
+  typedef float elem;
+  static constexpr int kPerVec = 4;
+  static __device__ __forceinline__ u32x4 add(u32x4 a, u32x4 b) {
+    u32x4 r;
+    r.x = __float_as_uint(__uint_as_float(a.x) + __uint_as_float(b.x));
+    r.y = __float_as_uint(__uint_as_float(a.y) + __uint_as_float(b.y));
+    r.z = __float_as_uint(__uint_as_float(a.z) + __uint_as_float(b.z));
+    r.w = __float_as_uint(__uint_as_float(a.w) + __uint_as_float(b.w));
+    return r;
+  }
+  static __device__ __forceinline__ elem add1(elem a, elem b) { return a + b; }
+};
+
+// Two bf16 values per 32-bit word, element 2i in the low half.
+struct OpBF16 {
+  typedef uint16_t elem;
+  static constexpr int kPerVec = 8;
+  static __device__ __forceinline__ uint32_t add_word(uint32_t a, uint32_t b) {
+    float lo = __uint_as_float(a << 16) + __uint_as_float(b << 16);
+    float hi = __uint_as_float(a & 0xffff0000u) + __uint_as_float(b & 0xffff0000u);
+    return (bf16_round_hi(lo) >> 16) | bf16_round_hi(hi);
+  }
+  static __device__ __forceinline__ u32x4 add(u32x4 a, u32x4 b) {
+    u32x4 r;
+    r.x = add_word(a.x, b.x);
+    r.y = add_word(a.y, b.y);
+    r.z = add_word(a.z, b.z);
+    r.w = add_word(a.w, b.w);
+    return r;
+  }
+  static __device__ __forceinline__ elem add1(elem a, elem b) {
+    float s = __uint_as_float((uint32_t)a << 16) + __uint_as_float((uint32_t)b << 16);
+    return (elem)(bf16_round_hi(s) >> 16);
+  }
+};
+
+// Partial sums of the fused reduce.  An accumulator is held as fp32 lanes; for
+// bf16 with per-hop rounding the fp32 value is re-rounded to bf16 precision
+// after every add, which is bit-identical to storing and re-loading bf16.
+struct AccF32 {
+  typedef OpF32 op;
+  static constexpr int kLanes = 4;   // fp32 lanes per 16-byte input vector
+  static __device__ __forceinline__ void widen(u32x4 v, float* f) {
+    f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y);
+    f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
+  }
+  static __device__ __forceinline__ float hop(float a, float b) { return a + b; }
+  static __device__ __forceinline__ u32x4 narrow(const float* f) {
+    u32x4 r;
+    r.x = __float_as_uint(f[0]); r.y = __float_as_uint(f[1]);
+    r.z = __float_as_uint(f[2]); r.w = __float_as_uint(f[3]);
+    return r;
+  }
+};
+
+template <bool PER_HOP>
+struct AccBF16 {
+  typedef OpBF16 op;
+  static constexpr int kLanes = 8;
+  static __device__ __forceinline__ void widen(u32x4 v, float* f) {
+    f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+    f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+    f[4] = __uint_as_float(v.z << 16); f[5] = __uint_as_float(v.z & 0xffff0000u);
+    f[6] = __uint_as_float(v.w << 16); f[7] = __uint_as_float(v.w & 0xffff0000u);
+  }
+  static __device__ __forceinline__ float hop(float a, float b) {
+    float s = a + b;
+    if constexpr (PER_HOP) return __uint_as_float(bf16_round_hi(s));
+    else return s;
+  }
+  static __device__ __forceinline__ u32x4 narrow(const float* f) {
+    u32x4 r;
+    r.x = (bf16_round_hi(f[0]) >> 16) | bf16_round_hi(f[1]);
+    r.y = (bf16_round_hi(f[2]) >> 16) | bf16_round_hi(f[3]);
+    r.z = (bf16_round_hi(f[4]) >> 16) | bf16_round_hi(f[5]);
+    r.w = (bf16_round_hi(f[6]) >> 16) | bf16_round_hi(f[7]);
+    return r;
+  }
+};
+
+// How a segment of `n` elements at (dst, a, b) splits into an unaligned head
+// (elements before the first 16-byte boundary), a body of whole 128-bit vectors
+// and a tail.  If the operands do not share one misalignment the whole segment
+// is done element by element (vec == 0).
+struct Split {
+  size_t head;   // elements
+  size_t vec;    // 16-byte vectors
+  size_t tail;   // elements
+};
+
+__device__ __forceinline__ Split split_segment(uintptr_t p0, uintptr_t p1, uintptr_t p2, size_t n,
+                                               unsigned esize) {
+  Split s;
+  unsigned mis = (unsigned)(p0 & 15u);
+  if ((p1 & 15u) != mis || (p2 & 15u) != mis || (mis % esize) != 0) {
+    s.head = n; s.vec = 0; s.tail = 0;
+    return s;
+  }
+  size_t head = ((16u - mis) & 15u) / esize;
+  if (head > n) head = n;
+  size_t per = 16u / esize;
+  s.head = head;
+  s.vec = (n - head) / per;
+  s.tail = n - head - s.vec * per;
+  if (s.vec == 0) { s.head = n; s.tail = 0; }
+  return s;
+}
+
+// dst = a + b over one tile of a segment.  Tile `tile` covers vectors
+// [tile*kThreads*U, (tile+1)*kThreads*U); tile 0 also does head and tail.
+template <class Op, int U, bool NTL, bool NTS>
+__device__ __forceinline__ void add_tile(void* dstp, const void* ap, const void* bp, size_t n,
+                                         size_t tile) {
+  typedef typename Op::elem elem;
+  const Split sp = split_segment((uintptr_t)dstp, (uintptr_t)ap, (uintptr_t)bp, n, sizeof(elem));
+  elem* de = (elem*)dstp;
+  const elem* ae = (const elem*)ap;
+  const elem* be = (const elem*)bp;
+  const unsigned tid = threadIdx.x;
+
+  if (sp.vec == 0) {
+    // no common alignment (or a segment shorter than one vector): scalar path,
+    // each tile takes the element range its vectors would have covered
+    const size_t per_tile = (size_t)kThreads * U * Op::kPerVec;
+    size_t lo = tile * per_tile;
+    size_t hi = lo + per_tile < sp.head ? lo + per_tile : sp.head;
+    for (size_t i = lo + tid; i < hi; i += kThreads) de[i] = Op::add1(ae[i], be[i]);
+    return;
+  }
+
+  u32x4* dv = (u32x4*)(de + sp.head);
+  const u32x4* av = (const u32x4*)(ae + sp.head);
+  const u32x4* bv = (const u32x4*)(be + sp.head);
+  const size_t base = tile * (size_t)(kThreads * U);
+
+  if (base + (size_t)kThreads * U <= sp.vec) {
+    u32x4 x[U], y[U];
+#pragma unroll
+    for (int j = 0; j < U; ++j) x[j] = ld16<NTL>(av + base + (size_t)j * kThreads + tid);
+#pragma unroll
+    for (int j = 0; j < U; ++j) y[j] = ld16<NTL>(bv + base + (size_t)j * kThreads + tid);
+#pragma unroll
+    for (int j = 0; j < U; ++j) st16<NTS>(dv + base + (size_t)j * kThreads + tid, Op::add(x[j], y[j]));
+  } else {
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      size_t v = base + (size_t)j * kThreads + tid;
+      if (v < sp.vec) st16<NTS>(dv + v, Op::add(ld16<NTL>(av + v), ld16<NTL>(bv + v)));
+    }
+  }
+
+  if (tile == 0) {
+    if (tid < sp.head) de[tid] = Op::add1(ae[tid], be[tid]);
+    if (tid >= 64 && tid - 64 < sp.tail) {
+      size_t i = sp.head + sp.vec * Op::kPerVec + (tid - 64);
+      de[i] = Op::add1(ae[i], be[i]);
+    }
+  }
+}
+
+// Byte copy of one tile of a segment (same splitting, element = byte).
+template <int U, bool NTL, bool NTS>
+__device__ __forceinline__ void copy_tile(void* dstp, const void* srcp, size_t nbytes, size_t tile) {
+  const Split sp = split_segment((uintptr_t)dstp, (uintptr_t)srcp, (uintptr_t)srcp, nbytes, 1);
+  uint8_t* d8 = (uint8_t*)dstp;
+  const uint8_t* s8 = (const uint8_t*)srcp;
+  const unsigned tid = threadIdx.x;
+
+  if (sp.vec == 0) {
+    const size_t per_tile = (size_t)kThreads * U * 16;
+    size_t lo = tile * per_tile;
+    if (lo >= sp.head) return;
+    size_t hi = lo + per_tile < sp.head ? lo + per_tile : sp.head;
+    if ((((uintptr_t)dstp | (uintptr_t)srcp) & 3u) == 0) {
+      // both 4-byte aligned: move words, then the last 0-3 bytes
+      size_t wlo = lo / 4, whi = hi / 4;
+      uint32_t* d32 = (uint32_t*)dstp;
+      const uint32_t* s32 = (const uint32_t*)srcp;
+      for (size_t i = wlo + tid; i < whi; i += kThreads) d32[i] = s32[i];
+      if (hi == sp.head) {
+        size_t i = whi * 4 + tid;
+        if (i < hi) d8[i] = s8[i];
+      }
+    } else {
+      for (size_t i = lo + tid; i < hi; i += kThreads) d8[i] = s8[i];
+    }
+    return;
+  }
+
+  u32x4* dv = (u32x4*)(d8 + sp.head);
+  const u32x4* sv = (const u32x4*)(s8 + sp.head);
+  const size_t base = tile * (size_t)(kThreads * U);
+  if (base + (size_t)kThreads * U <= sp.vec) {
+    u32x4 x[U];
+#pragma unroll
+    for (int j = 0; j < U; ++j) x[j] = ld16<NTL>(sv + base + (size_t)j * kThreads + tid);
+#pragma unroll
+    for (int j = 0; j < U; ++j) st16<NTS>(dv + base + (size_t)j * kThreads + tid, x[j]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      size_t v = base + (size_t)j * kThreads + tid;
+      if (v < sp.vec) st16<NTS>(dv + v, ld16<NTL>(sv + v));
+    }
+  }
+  if (tile == 0) {
+    if (tid < sp.head) d8[tid] = s8[tid];
+    if (tid >= 64 && tid - 64 < sp.tail) {
+      size_t i = sp.head + sp.vec * 16 + (tid - 64);
+      d8[i] = s8[i];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// kernels
+// ---------------------------------------------------------------------------
+struct AddSegs {
+  void* dst[kMaxSeg];
+  const void* a[kMaxSeg];
+  const void* b[kMaxSeg];
+};
+
+// `count` segments of n elements: dst[s] = a[s] + b[s].
+template <class Op, int U, bool NTL, bool NTS>
+__global__ __launch_bounds__(kThreads) void k_add_segs(AddSegs t, int count, size_t n,
+                                                       size_t tiles_per_seg) {
+  const size_t total = (size_t)count * tiles_per_seg;
+  for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
+    const int s = (int)(w / tiles_per_seg);
+    const size_t tile = w - (size_t)s * tiles_per_seg;
+    add_tile<Op, U, NTL, NTS>(t.dst[s], t.a[s], t.b[s], n, tile);
+  }
+}
+
+struct RhArgs {
+  void* bufs[kMaxSeg];
+  const void* src[kMaxSeg];
+  void* outs[kMaxSeg];
+};
+
+// One recursive-halving round for all P ranks: the strided-half pairwise add.
+// Rank r and its partner own the same active region [start, start + 2*count);
+// the lower rank of the pair sums the lower halves into its buffer, the upper
+// rank the upper halves into its own.
+template <class Op, int U, bool NTL, bool NTS>
+__global__ __launch_bounds__(kThreads) void k_rh_round(RhArgs t, int P, size_t B, int round,
+                                                       int from_src, int to_outs,
+                                                       size_t tiles_per_seg) {
+  typedef typename Op::elem elem;
+  const int group = P >> round;
+  const int half = group >> 1;
+  const size_t count = (size_t)half * B;
+  const size_t total = (size_t)P * tiles_per_seg;
+  for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
+    const int r = (int)(w / tiles_per_seg);
+    const size_t tile = w - (size_t)r * tiles_per_seg;
+    const bool lower = (r % group) < half;
+    const int partner = lower ? r + half : r - half;
+    const size_t off = (size_t)(r / group) * group * B + (lower ? 0 : count);
+    const elem* a = (const elem*)(from_src ? t.src[r] : t.bufs[r]) + off;
+    const elem* b = (const elem*)(from_src ? t.src[partner] : t.bufs[partner]) + off;
+    elem* d = to_outs ? (elem*)t.outs[r] : (elem*)t.bufs[r] + off;
+    add_tile<Op, U, NTL, NTS>(d, a, b, count, tile);
+  }
+}
+
+struct CopySegs {
+  void* dst[kMaxSeg];
+  const void* src[kMaxSeg];
+  size_t nbytes[kMaxSeg];
+};
+
+// `count` byte segments; tiles_per_seg is sized for the longest one.
+template <int U, bool NTL, bool NTS>
+__global__ __launch_bounds__(kThreads) void k_copy_segs(CopySegs t, int count,
+                                                        size_t tiles_per_seg) {
+  const size_t total = (size_t)count * tiles_per_seg;
+  const size_t tile_bytes = (size_t)kThreads * U * 16;
+  for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
+    const int s = (int)(w / tiles_per_seg);
+    const size_t tile = w - (size_t)s * tiles_per_seg;
+    const size_t nb = t.nbytes[s];
+    // a tile past the end of a short segment has nothing to do (16 spare
+    // bytes cover the head shift of the vector body)
+    if (tile != 0 && tile * tile_bytes >= nb + 16) continue;
+    copy_tile<U, NTL, NTS>(t.dst[s], t.src[s], nb, tile);
+  }
+}
+
+struct GatherArgs {
+  void* outs[kMaxSeg];
+  const void* ins[kMaxSeg];
+  size_t nbytes[kMaxSeg];
+  size_t dst_off[kMaxSeg];
+};
+
+// Direct all_gather placement for all P ranks: a workgroup reads one tile of
+// shard k ONCE and stores it into every rank's output at dst_off[k], so the
+// shards are fetched from HBM once instead of P times.
+template <int U, bool NTL, bool NTS>
+__global__ __launch_bounds__(kThreads) void k_gather_multicast(GatherArgs t, int P, int nout,
+                                                              size_t tiles_per_seg) {
+  const size_t total = (size_t)P * tiles_per_seg;
+  const size_t tile_bytes = (size_t)kThreads * U * 16;
+  const unsigned tid = threadIdx.x;
+  for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
+    const int k = (int)(w / tiles_per_seg);
+    const size_t tile = w - (size_t)k * tiles_per_seg;
+    const size_t nb = t.nbytes[k];
+    if (tile != 0 && tile * tile_bytes >= nb + 16) continue;
+    const uint8_t* src = (const uint8_t*)t.ins[k];
+    const size_t off = t.dst_off[k];
+    // vector path only if the source and EVERY destination share alignment
+    bool aligned = ((uintptr_t)src & 15u) == 0 && (off & 15u) == 0;
+    for (int r = 0; r < nout; ++r) aligned = aligned && (((uintptr_t)t.outs[r]) & 15u) == 0;
+    const size_t nvec = nb / 16;
+    const size_t base = tile * (size_t)(kThreads * U);
+    if (aligned && base + (size_t)kThreads * U <= nvec) {
+      const u32x4* sv = (const u32x4*)src;
+      u32x4 x[U];
+#pragma unroll
+      for (int j = 0; j < U; ++j) x[j] = ld16<NTL>(sv + base + (size_t)j * kThreads + tid);
+      for (int r = 0; r < nout; ++r) {
+        u32x4* dv = (u32x4*)((uint8_t*)t.outs[r] + off);
+#pragma unroll
+        for (int j = 0; j < U; ++j) st16<NTS>(dv + base + (size_t)j * kThreads + tid, x[j]);
+      }
+    } else {
+      for (int r = 0; r < nout; ++r)
+        copy_tile<U, NTL, NTS>((uint8_t*)t.outs[r] + off, src, nb, tile);
+    }
+  }
+}
+
+// dst[c][r][0:m] = src[r][c][0:m] (bytes): the 2-D block transpose.
+template <int U, bool NTL, bool NTS>
+__global__ __launch_bounds__(kThreads) void k_block_transpose(uint8_t* dst, const uint8_t* src,
+                                                              size_t rows, size_t cols, size_t m,
+                                                              size_t tiles_per_seg) {
+  const size_t total = rows * cols * tiles_per_seg;
+  for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
+    const size_t blk = w / tiles_per_seg;            // destination block index c*rows + r
+    const size_t tile = w - blk * tiles_per_seg;
+    const size_t c = blk / rows, r = blk - c * rows;
+    copy_tile<U, NTL, NTS>(dst + blk * m, src + (r * cols + c) * m, m, tile);
+  }
+}
+
+struct KwayArgs {
+  const void* shard[kMaxSeg];
+  void* out[kMaxSeg];
+};
+
+// S(M, H) of the halving butterfly over K leaves v[m] = shard[first ^ m]:
+// S(M, K) = v[M];  S(M, H) = S(M, 2H) + S(M + H, 2H);  the result is S(0, 1).
+// Unfolding v[m] += v[m+h] for h = K/2 .. 1 gives exactly this tree.  Every
+// index is a template constant, so partial sums live in registers.
+template <class Acc, int K, int M, int H, int L, class Load>
+__device__ __forceinline__ void tree_sum(Load& load, int first, float* out) {
+  if constexpr (H == K) {
+    load(first ^ M, out);
+  } else {
+    float lo[L], hi[L];
+    tree_sum<Acc, K, M, 2 * H, L>(load, first, lo);
+    tree_sum<Acc, K, M + H, 2 * H, L>(load, first, hi);
+#pragma unroll
+    for (int l = 0; l < L; ++l) out[l] = Acc::hop(lo[l], hi[l]);
+  }
+}
+
+// Fold the k shards at one position in the order of a schedule.
+//   K == 0 : ring order, runtime k: first, first+1, ... (mod k), loads issued
+//            in batches of four ahead of the adds
+//   K >= 2 : halving order for k == K: leaves v[m] = shard[first ^ m] summed by
+//            the butterfly v[m] += v[m+h], h = K/2 .. 1, evaluated depth first
+//            by tree_sum (the same tree with only log2 K live partial sums).
+// load(q, f) fills the L fp32 lanes of shard q; acc receives the result.
+template <class Acc, int K, int L, class Load>
+__device__ __forceinline__ void fold_shards(Load&& load, int k, int first, float* acc) {
+  if constexpr (K == 0) {
+    int q = first;
+    load(q, acc);
+    int done = 1;
+    for (; done + 4 <= k; done += 4) {
+      float f[4][L];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        q = q + 1 == k ? 0 : q + 1;
+        load(q, f[i]);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int l = 0; l < L; ++l) acc[l] = Acc::hop(acc[l], f[i][l]);
+    }
+    for (; done < k; ++done) {
+      q = q + 1 == k ? 0 : q + 1;
+      float f[L];
+      load(q, f);
+#pragma unroll
+      for (int l = 0; l < L; ++l) acc[l] = Acc::hop(acc[l], f[l]);
+    }
+  } else {
+    tree_sum<Acc, K, 0, 1, L>(load, first, acc);
+  }
+}
+
+// Fused k-way reduce, one pass: output j = fold over the k shards of
+// shard[.][j*stride + i], i < n, starting the schedule at shard
+// (first0 + j) mod k.  The vector path needs 16-byte aligned operands;
+// otherwise (and for the last n % kPerVec elements) elements go one by one
+// through the same fold.
+template <class Acc, int K, int U, bool NTL, bool NTS>
+__global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int nout,
+                                                          size_t stride, size_t n, int first0,
+                                                          size_t tiles_per_seg) {
+  typedef typename Acc::op Op;
+  typedef typename Op::elem elem;
+  constexpr int L = Acc::kLanes;
+  const size_t total = (size_t)nout * tiles_per_seg;
+  const unsigned tid = threadIdx.x;
+  for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
+    const int j = (int)(w / tiles_per_seg);
+    const size_t tile = w - (size_t)j * tiles_per_seg;
+    const int first = (first0 + j) % k;
+    const size_t eoff = (size_t)j * stride;
+    elem* out = (elem*)t.out[j];
+
+    bool aligned = (((uintptr_t)out) & 15u) == 0;
+    for (int q = 0; q < k; ++q)
+      aligned = aligned && (((uintptr_t)((const elem*)t.shard[q] + eoff)) & 15u) == 0;
+    const size_t nvec = aligned ? n / Op::kPerVec : 0;
+    const size_t base = tile * (size_t)(kThreads * U);
+
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const size_t v = base + (size_t)u * kThreads + tid;
+      if (v < nvec) {
+        float acc[L];
+        fold_shards<Acc, K, L>(
+            [&](int q, float* f) {
+              Acc::widen(ld16<NTL>((const u32x4*)((const elem*)t.shard[q] + eoff) + v), f);
+            },
+            k, first, acc);
+        st16<NTS>((u32x4*)out + v, Acc::narrow(acc));
+      }
+    }
+
+    // scalar remainder: the tail of an aligned segment (tile 0), or everything
+    size_t lo, hi;
+    if (aligned) {
+      lo = nvec * Op::kPerVec;
+      hi = tile == 0 ? n : lo;
+    } else {
+      const size_t per_tile = (size_t)kThreads * U * Op::kPerVec;
+      lo = tile * per_tile;
+      hi = lo + per_tile < n ? lo + per_tile : n;
+    }
+    for (size_t i = lo + tid; i < hi; i += kThreads) {
+      float acc1[1];
+      fold_shards<Acc, K, 1>(
+          [&](int q, float* f) {
+            elem e = ((const elem*)t.shard[q] + eoff)[i];
+            if constexpr (sizeof(elem) == 4) f[0] = e;
+            else f[0] = __uint_as_float((uint32_t)e << 16);
+          },
+          k, first, acc1);
+      if constexpr (sizeof(elem) == 4) out[i] = acc1[0];
+      else out[i] = (elem)(bf16_round_hi(acc1[0]) >> 16);
+    }
+  }
+}
+
+}  // namespace pccl_kernels
+
+#endif  // PCCL_KERNELS_H

@@ -1,0 +1,279 @@
+"""Torch-facing wrappers of the HIP kernels in libpccl_hip.so.
+
+PyTorch-ROCm is used for what the reference uses it for: device memory and the
+current stream (pccl/src/reduce_scatter.cpp:29,116; pccl/src/all_gather.cpp:28).
+Every function validates its tensors on the host, takes raw device addresses
+and enqueues on `torch.cuda.current_stream()`.  Nothing here computes on the
+CPU: tensors that are not on the GPU are rejected.
+"""
+from __future__ import annotations
+
+import os
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import _native
+from ._native import (BF16, F32, MODE_FAITHFUL, MODE_FUSED, MODE_STEPS, ORDER_HALVING,
+                      ORDER_RING, MAX_RANKS)
+
+_MODES = {"steps": MODE_STEPS, "fused": MODE_FUSED, "faithful": MODE_FAITHFUL}
+
+
+def mode_code(mode) -> int:
+    """'steps' | 'fused' | 'faithful' (or None = $PCCL_VIRTUAL_MODE, default steps)."""
+    if mode is None:
+        mode = os.environ.get("PCCL_VIRTUAL_MODE", "steps")
+    if isinstance(mode, int):
+        if mode not in _MODES.values():
+            raise ValueError(f"unknown mode {mode}")
+        return mode
+    try:
+        return _MODES[str(mode)]
+    except KeyError:
+        raise ValueError(f"unknown mode {mode!r}; expected one of {sorted(_MODES)}") from None
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    """Element type of the reduction kernels.  The reference's extension takes
+    float32 only (pccl/src/pccl.cpp:42-45); bfloat16 is what its Python
+    algorithms add with torch.add."""
+    if dtype == torch.float32:
+        return F32
+    if dtype == torch.bfloat16:
+        return BF16
+    raise RuntimeError("Input tensor must be of type float (float32 or bfloat16)")
+
+
+def stream_handle() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def check_device_tensor(t: torch.Tensor, name: str):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must reside on the GPU (got device {t.device}); "
+                           "the HIP kernels have no CPU fallback")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} tensor must be contiguous.")
+
+
+def _same_device(tensors: Sequence[torch.Tensor]):
+    dev = tensors[0].device
+    for t in tensors:
+        if t.device != dev:
+            raise RuntimeError("all virtual ranks must live on one GPU")
+
+
+def _ptrs(tensors: Optional[Sequence[torch.Tensor]]):
+    return None if tensors is None else [t.data_ptr() for t in tensors]
+
+
+# ---------------------------------------------------------------------------
+# element kernels
+# ---------------------------------------------------------------------------
+
+def accumulate(dst: torch.Tensor, src: torch.Tensor):
+    """dst += src  (pccl/src/common.cu:5-19)."""
+    check_device_tensor(dst, "dst"); check_device_tensor(src, "src")
+    if dst.dtype != src.dtype or dst.numel() != src.numel():
+        raise RuntimeError("accumulate: dst and src must have the same dtype and size")
+    _native.load().accumulate(dst.data_ptr(), src.data_ptr(), dst.numel(), dtype_code(dst.dtype),
+                              stream_handle())
+
+
+def add(dst: torch.Tensor, a: torch.Tensor, b: torch.Tensor):
+    """dst = a + b (dst may be a or b)."""
+    for t, n in ((dst, "dst"), (a, "a"), (b, "b")):
+        check_device_tensor(t, n)
+    if not (dst.dtype == a.dtype == b.dtype) or not (dst.numel() == a.numel() == b.numel()):
+        raise RuntimeError("add: operands must have the same dtype and size")
+    _native.load().add(dst.data_ptr(), a.data_ptr(), b.data_ptr(), dst.numel(), dtype_code(dst.dtype),
+                       stream_handle())
+
+
+def add_batched(dst: Sequence[torch.Tensor], a: Sequence[torch.Tensor], b: Sequence[torch.Tensor]):
+    """dst[s] = a[s] + b[s] for every segment s in one launch."""
+    if not (len(dst) == len(a) == len(b)):
+        raise ValueError("dst, a, b must have the same number of segments")
+    if not dst:
+        return
+    n, dt = dst[0].numel(), dst[0].dtype
+    for group, nm in ((dst, "dst"), (a, "a"), (b, "b")):
+        for t in group:
+            check_device_tensor(t, nm)
+            if t.numel() != n or t.dtype != dt:
+                raise RuntimeError("add_batched: all segments must have the same dtype and size")
+    _native.load().add_batched(_ptrs(dst), _ptrs(a), _ptrs(b), n, dtype_code(dt), stream_handle())
+
+
+def copy(dst: torch.Tensor, src: torch.Tensor):
+    """Byte copy dst <- src (same number of bytes)."""
+    copy_batched([dst], [src])
+
+
+def copy_batched(dst: Sequence[torch.Tensor], src: Sequence[torch.Tensor]):
+    """dst[s] <- src[s] (bytes) for every segment in one launch."""
+    if len(dst) != len(src):
+        raise ValueError("dst and src must have the same number of segments")
+    nbytes = []
+    for d, s in zip(dst, src):
+        check_device_tensor(d, "dst"); check_device_tensor(s, "src")
+        nb = d.numel() * d.element_size()
+        if nb != s.numel() * s.element_size():
+            raise RuntimeError("copy_batched: segment sizes differ")
+        nbytes.append(nb)
+    lib = _native.load()
+    for i in range(0, len(dst), MAX_RANKS):
+        lib.copy_batched(_ptrs(dst[i:i + MAX_RANKS]), _ptrs(src[i:i + MAX_RANKS]),
+                         nbytes[i:i + MAX_RANKS], stream_handle())
+
+
+def reduce_kway(out: torch.Tensor, shards: Sequence[torch.Tensor], order: str = "ring", first: int = 0,
+                per_hop_round: bool = True):
+    """out = sum of the shards, added in the order of a schedule, in one pass.
+
+    order 'ring': shards first, first+1, ... (mod k) as a left fold;
+    order 'halving': the butterfly of recursive halving rooted at `first`."""
+    check_device_tensor(out, "out")
+    for s in shards:
+        check_device_tensor(s, "shard")
+        if s.dtype != out.dtype or s.numel() != out.numel():
+            raise RuntimeError("reduce_kway: shards must match the output's dtype and size")
+    code = {"ring": ORDER_RING, "halving": ORDER_HALVING}.get(order)
+    if code is None:
+        raise ValueError(f"unknown order {order!r}")
+    _native.load().reduce_kway(out.data_ptr(), _ptrs(shards), out.numel(), dtype_code(out.dtype), code,
+                               first, per_hop_round, stream_handle())
+
+
+def block_transpose(dst: torch.Tensor, src: torch.Tensor, rows: int, cols: int):
+    """dst = src.view(rows, cols, -1).transpose(0, 1).reshape(-1)
+    (pccl/reduce_scatter.py:226, pccl/all_gather.py:158)."""
+    check_device_tensor(dst, "dst"); check_device_tensor(src, "src")
+    nb = src.numel() * src.element_size()
+    if dst.numel() * dst.element_size() != nb or dst.dtype != src.dtype:
+        raise RuntimeError("block_transpose: dst and src must have the same dtype and size")
+    if rows * cols == 0 or src.numel() % (rows * cols):
+        raise RuntimeError("block_transpose: size must be divisible by rows*cols")
+    if dst.data_ptr() == src.data_ptr() and nb:
+        raise RuntimeError("block_transpose: dst must not alias src")
+    _native.load().block_transpose(dst.data_ptr(), src.data_ptr(), rows, cols, nb // (rows * cols),
+                                   stream_handle())
+
+
+# ---------------------------------------------------------------------------
+# whole collectives over a list of virtual ranks (group-rank order)
+# ---------------------------------------------------------------------------
+
+def reduce_scatter_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[torch.Tensor],
+                         algorithm: str = "ring", mode=None,
+                         work: Optional[Sequence[torch.Tensor]] = None) -> None:
+    """reduce_scatter over P = len(inputs) virtual ranks in one call.
+
+    inputs[r] holds P*B elements, outputs[r] receives block r of the sum with
+    the summation order of `algorithm` ('ring': pccl/src/reduce_scatter.cpp:101-155,
+    'recursive': :16-99).  Workspaces are taken from torch's caching allocator
+    when the mode needs them, as the reference's shim does (pccl/src/pccl.cpp:58-73)."""
+    P = len(inputs)
+    if len(outputs) != P or P < 1:
+        raise ValueError("need one output per input rank")
+    if P > MAX_RANKS:
+        raise RuntimeError(f"at most {MAX_RANKS} virtual ranks per communicator")
+    for t in inputs:
+        check_device_tensor(t, "input")
+    for t in outputs:
+        check_device_tensor(t, "output")
+    _same_device(list(inputs) + list(outputs))
+    total = inputs[0].numel()
+    dt = inputs[0].dtype
+    if total % P:
+        raise RuntimeError("Input tensor size must be divisible by number of processes")
+    B = total // P
+    for i, o in zip(inputs, outputs):
+        if i.numel() != total or i.dtype != dt:
+            raise RuntimeError("all ranks must pass inputs of the same dtype and size")
+        if o.numel() != B:
+            raise RuntimeError("Output tensor must have block_size elements (input tensor numel()/world_size)")
+        if o.dtype != dt:
+            raise RuntimeError("Output tensor must be of type float (same dtype as the input)")
+    m = mode_code(mode)
+    need_work = (m == MODE_FAITHFUL and P > 1) or (m == MODE_STEPS and P > 2)
+    if need_work and work is None:
+        work = [torch.empty_like(inputs[r]) for r in range(P)]
+    if work is not None:
+        for w in work:
+            check_device_tensor(w, "work")
+            if w.numel() < total or w.dtype != dt:
+                raise RuntimeError("work buffers must have the input's dtype and size")
+    _native.load().reduce_scatter_virtual(_ptrs(outputs), _ptrs(inputs), _ptrs(work) if need_work else None,
+                                          B, dtype_code(dt), algorithm, m, stream_handle())
+
+
+def all_gather_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[torch.Tensor],
+                     algorithm: str = "recursive", mode=None) -> None:
+    """all_gather over P virtual ranks: outputs[r] = cat(inputs) for every r
+    ('recursive': pccl/src/all_gather.cpp:15-69; 'ring': this build's schedule)."""
+    P = len(inputs)
+    if len(outputs) != P or P < 1:
+        raise ValueError("need one output per input rank")
+    if P > MAX_RANKS:
+        raise RuntimeError(f"at most {MAX_RANKS} virtual ranks per communicator")
+    for t in inputs:
+        check_device_tensor(t, "input")
+    for t in outputs:
+        check_device_tensor(t, "output")
+    _same_device(list(inputs) + list(outputs))
+    blk = inputs[0].numel()
+    dt = inputs[0].dtype
+    for i, o in zip(inputs, outputs):
+        if i.numel() != blk or i.dtype != dt:
+            raise RuntimeError("all ranks must pass shards of the same dtype and size")
+        if o.dtype != dt:
+            raise RuntimeError("Input and output tensors must have the same dtype.")
+        if o.numel() != blk * P:
+            raise RuntimeError("Output tensor must have total_elem elements (input tensor numel() *world_size)")
+    _native.load().all_gather_virtual(_ptrs(outputs), _ptrs(inputs), blk * inputs[0].element_size(),
+                                      algorithm, mode_code(mode), stream_handle())
+
+
+def padded_offsets(nbytes: Sequence[int], align: int = 256) -> List[int]:
+    """Byte offset of each shard when every shard is padded to `align` bytes."""
+    off, out = 0, []
+    for nb in nbytes:
+        out.append(off)
+        off += (nb + align - 1) // align * align
+    return out
+
+
+def all_gather_uneven_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[torch.Tensor],
+                            dst_off: Optional[Sequence[int]] = None, align: int = 256) -> List[int]:
+    """all_gather of shards of different lengths: shard k lands at byte offset
+    dst_off[k] (default: each shard padded to `align` bytes) of every output.
+    Bytes between shards are left untouched.  Returns the offsets used.
+    Not a reference feature (it requires equal shards, pccl/src/pccl.cpp:111-116)."""
+    P = len(inputs)
+    if len(outputs) != P or P < 1:
+        raise ValueError("need one output per input rank")
+    for t in inputs:
+        check_device_tensor(t, "input")
+    for t in outputs:
+        check_device_tensor(t, "output")
+    _same_device(list(inputs) + list(outputs))
+    nbytes = [t.numel() * t.element_size() for t in inputs]
+    if dst_off is None:
+        dst_off = padded_offsets(nbytes, align)
+    if len(dst_off) != P:
+        raise ValueError("need one offset per shard")
+    spans = sorted((int(o), int(o) + nb) for o, nb in zip(dst_off, nbytes))
+    for (_, e0), (s1, _) in zip(spans, spans[1:]):
+        if s1 < e0:
+            raise RuntimeError("all_gather_uneven: shards overlap in the output")
+    end = max((int(o) + nb for o, nb in zip(dst_off, nbytes)), default=0)
+    for o in outputs:
+        if o.numel() * o.element_size() < end:
+            raise RuntimeError("all_gather_uneven: output too small for the shard layout")
+    _native.load().all_gather_uneven_virtual(_ptrs(outputs), _ptrs(inputs), nbytes, list(dst_off),
+                                             stream_handle())
+    return list(dst_off)
