@@ -1,0 +1,395 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-GPU reduce/copy kernels of PCCL's collectives on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--mode M]
+
+Prints ONE JSON line.  A "step" is one whole collective over the virtual ranks
+of the workload with all inputs already resident in HBM; `value` is the
+algorithmic bytes of that collective divided by its time (GB/s, 1 GB = 1e9 B).
+Timing follows benchmark_raw_collectives/utils.py:16-33 of the reference:
+warm-up calls, then the mean over the timed calls between two device events.
+
+Workloads (BASELINE.json `configs`; `cfg2` is the one the metric is quoted on):
+  cfg1  ring reduce_scatter, P=4, fp32, 16 Mi elements per rank
+  cfg2  ring reduce_scatter, P=8, bf16, 256 Mi elements per rank, per-hop
+        accumulate with bf16 rounding at every hop              (default)
+  cfg3  recursive-halving round at its largest shape: a pair of ranks adding
+        512 MiB strided halves (bf16), i.e. round 0 of P=64 with 1 GiB per rank
+  cfg4  all_gather placement, P=16, bf16 shards of 128 MiB into 2 GiB outputs
+  cfg4u the same with uneven shards padded to 256 bytes
+  cfg5  fused one-pass reduce of 32 fp32 shards of 32 Mi elements
+
+The CPU baseline (the reference's per-rank algorithm on host cores, one process
+per rank over MPI_Sendrecv, or fork+shared memory where no MPI launcher
+exists) is timed on a bounded sample and reported beside the GPU number; it is
+a baseline, not a target.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import shutil
+import subprocess
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "sc2025-pccl-reproducer_amd"))
+
+METRIC = "reduce/copy kernel HBM GB/s and % of MI355X peak at 64MB-2GB messages"
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
+MiB = 1 << 20
+
+
+def parse_args():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="cfg2",
+                    choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg4u", "cfg5"])
+    ap.add_argument("--mode", default=None, choices=["steps", "fused", "faithful"],
+                    help="execution mode of the collective (default: per-step replay)")
+    ap.add_argument("--scale", type=float, default=1.0,
+                    help="shrink the per-rank message by this factor (1.0 = BASELINE size)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-verify", action="store_true")
+    ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
+                    help="launch tuning of the library (grid_cap, unroll, nt_load, nt_store)")
+    return ap.parse_args()
+
+
+# ---------------------------------------------------------------------------
+# workloads: each returns (run_step, info) with inputs resident on the GPU
+# ---------------------------------------------------------------------------
+
+def _randn_bf16(n, std, seed, device):
+    import torch
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    out = torch.empty(n, dtype=torch.bfloat16, device=device)
+    chunk = 1 << 26
+    for i in range(0, n, chunk):      # bounded fp32 temporaries
+        m = min(chunk, n - i)
+        out[i:i + m] = (torch.randn(m, generator=g, device=device) * std).to(torch.bfloat16)
+    return out
+
+
+def _rand_f32(n, seed, device, uniform=True):
+    import torch
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    if uniform:
+        return torch.rand(n, generator=g, device=device) * 2 - 1
+    return torch.randn(n, generator=g, device=device)
+
+
+def make_ring_rs(P, elems_per_rank, dtype, mode, device, seed=1234, std=1.0):
+    import torch
+    from pccl import kernels
+    B = elems_per_rank // P
+    total = B * P
+    if dtype == "bf16":
+        ins = [_randn_bf16(total, std, seed + r, device) for r in range(P)]
+        es = 2
+    else:
+        ins = [_rand_f32(total, seed + r, device) for r in range(P)]
+        es = 4
+    outs = [torch.empty(B, dtype=ins[0].dtype, device=device) for _ in range(P)]
+    m = kernels.mode_code(mode)
+    work = [torch.empty_like(ins[r]) for r in range(P)] if m != kernels.MODE_FUSED and P > 2 else None
+
+    def step():
+        kernels.reduce_scatter_ranks(outs, ins, "ring", m, work)
+
+    def verify():
+        # the three execution modes must agree bit for bit
+        ref = [torch.empty_like(o) for o in outs]
+        other = kernels.MODE_FUSED if m != kernels.MODE_FUSED else kernels.MODE_STEPS
+        w2 = work if work is not None else [torch.empty_like(ins[r]) for r in range(P)]
+        kernels.reduce_scatter_ranks(ref, ins, "ring", other, w2)
+        torch.cuda.synchronize()
+        return all(torch.equal(a.view(torch.uint8), b.view(torch.uint8)) for a, b in zip(outs, ref))
+
+    launches = {kernels.MODE_STEPS: P - 1, kernels.MODE_FUSED: 1, kernels.MODE_FAITHFUL: P + 1}[m]
+    if m == kernels.MODE_FUSED:
+        kernel_bytes = (P * P + P) * B * es             # reads every input once, writes every output
+        alg_bytes = kernel_bytes
+        kernel = "k_reduce_kway"
+    else:
+        kernel_bytes = 3 * P * B * es                   # one batched step: 2 reads + 1 write per rank
+        alg_bytes = (P - 1) * kernel_bytes
+        kernel = "k_add_segs"
+    info = dict(alg_bytes=alg_bytes, kernel=kernel, kernel_bytes=kernel_bytes,
+                kernel_launches=(P - 1 if m != kernels.MODE_FUSED else 1), launches=launches,
+                desc=f"ring reduce_scatter, P={P} virtual ranks, {dtype}, {total} elements per rank "
+                     f"({total * es / MiB:.0f} MiB), block {B} elements, mode={_mode_name(m)}",
+                dtype=dtype, P=P, B=B, verify=verify)
+    return step, info
+
+
+def _mode_name(m):
+    return {0: "steps", 1: "fused", 2: "faithful"}[m]
+
+
+def make_rh_pair(count_elems, device, seed=7):
+    """Round 0 of recursive halving at P=64 with 1 GiB per rank, seen by one
+    pair of ranks: P=2 here with B = count, so each rank adds one half."""
+    import torch
+    from pccl import _native, kernels
+    B = count_elems
+    ins = [_randn_bf16(2 * B, 1.0, seed + r, device) for r in range(2)]
+    work = [t.clone() for t in ins]
+    lib = _native.load()
+
+    def step():
+        lib.rh_round([w.data_ptr() for w in work], None, None, 2, B, 0, _native.BF16, kernels.stream_handle())
+
+    def verify():
+        # in place on the work buffers: redo once from the inputs and compare with torch
+        for w, i in zip(work, ins):
+            w.copy_(i)
+        step()
+        torch.cuda.synchronize()
+        n = min(B, 1 << 24)
+        lo = (ins[0][:n].float() + ins[1][:n].float()).bfloat16()
+        hi = (ins[1][B:B + n].float() + ins[0][B:B + n].float()).bfloat16()
+        return torch.equal(work[0][:n], lo) and torch.equal(work[1][B:B + n], hi)
+
+    kb = 2 * 3 * B * 2
+    info = dict(alg_bytes=kb, kernel="k_rh_round", kernel_bytes=kb, kernel_launches=1, launches=1,
+                desc=f"recursive-halving round, one pair of ranks, bf16, halves of {B * 2 / MiB:.0f} MiB "
+                     f"(round 0 of P=64 with {4 * B / MiB:.0f} MiB per rank)",
+                dtype="bf16", P=2, B=B, verify=verify)
+    return step, info
+
+
+def make_all_gather(P, shard_bytes, mode, device, uneven=False, seed=3):
+    import torch
+    from pccl import kernels
+    n = shard_bytes // 2
+    if uneven:
+        g = torch.Generator().manual_seed(seed)
+        lens = [int(n - int(torch.randint(0, n // 8, (1,), generator=g))) for _ in range(P)]
+    else:
+        lens = [n] * P
+    ins = [_randn_bf16(l, 1.0, seed + r, device) for r, l in enumerate(lens)]
+    nbytes = [2 * l for l in lens]
+    off = kernels.padded_offsets(nbytes, 256) if uneven else [r * shard_bytes for r in range(P)]
+    total = off[-1] + (nbytes[-1] + 255) // 256 * 256 if uneven else P * shard_bytes
+    outs = [torch.empty(total // 2, dtype=torch.bfloat16, device=device) for _ in range(P)]
+    m = kernels.mode_code(mode if mode else "fused")
+
+    if uneven:
+        def step():
+            kernels.all_gather_uneven_ranks(outs, ins, off)
+        launches, kernel = 1, "k_gather_multicast"
+    else:
+        def step():
+            kernels.all_gather_ranks(outs, ins, "ring", m)
+        launches = 1 if m == kernels.MODE_FUSED else P
+        kernel = "k_gather_multicast" if m == kernels.MODE_FUSED else "k_copy_segs"
+
+    def verify():
+        cat = torch.cat([t.view(torch.uint8) for t in ins]) if not uneven else None
+        for o in (outs[0], outs[P - 1]):
+            ob = o.view(torch.uint8)
+            if uneven:
+                for k in range(P):
+                    if not torch.equal(ob[off[k]:off[k] + nbytes[k]], ins[k].view(torch.uint8)):
+                        return False
+            elif not torch.equal(ob, cat):
+                return False
+        return True
+
+    payload = sum(nbytes)
+    alg = 2 * payload * P                       # 2 * bytes per materialised output, P outputs
+    if kernel == "k_gather_multicast":
+        kb, kl = alg, 1
+    else:
+        kb, kl = 2 * P * shard_bytes, P         # one batched step moves one shard per rank
+    info = dict(alg_bytes=alg, kernel=kernel, kernel_bytes=kb, kernel_launches=kl, launches=launches,
+                desc=f"all_gather placement, P={P} virtual ranks, bf16 shards of ~{shard_bytes / MiB:.0f} MiB"
+                     f"{' (uneven, padded to 256 B)' if uneven else ''} into {total / MiB:.0f} MiB outputs, "
+                     f"all {P} outputs materialised, mode={_mode_name(m) if not uneven else 'fused'}",
+                dtype="bf16", P=P, B=n, verify=verify)
+    return step, info
+
+
+def make_kway(k, n, device, seed=11):
+    import torch
+    from pccl import kernels
+    shards = [_rand_f32(n, seed + r, device, uniform=False) for r in range(k)]
+    out = torch.empty(n, device=device)
+
+    def step():
+        kernels.reduce_kway(out, shards, "ring", 1 % k)
+
+    def verify():
+        m = min(n, 1 << 22)
+        acc = shards[1 % k][:m].clone()
+        for t in range(1, k):
+            acc += shards[(1 + t) % k][:m]
+        return torch.equal(out[:m], acc)
+
+    kb = (k + 1) * n * 4
+    info = dict(alg_bytes=kb, kernel="k_reduce_kway", kernel_bytes=kb, kernel_launches=1, launches=1,
+                desc=f"fused one-pass reduce of {k} fp32 shards of {n} elements ({n * 4 / MiB:.0f} MiB each), "
+                     f"ring order", dtype="f32", P=k, B=n, verify=verify)
+    return step, info
+
+
+def build_workload(name, mode, scale, device):
+    def sc(x, q=1024):
+        return max(q, int(x * scale) // q * q)
+    if name == "cfg1":
+        return make_ring_rs(4, sc(16 * MiB), "f32", mode, device)
+    if name == "cfg2":
+        return make_ring_rs(8, sc(256 * MiB), "bf16", mode, device, std=1e-2)
+    if name == "cfg3":
+        return make_rh_pair(sc(256 * MiB), device)
+    if name == "cfg4":
+        return make_all_gather(16, sc(128 * MiB), mode, device)
+    if name == "cfg4u":
+        return make_all_gather(16, sc(128 * MiB), mode, device, uneven=True)
+    if name == "cfg5":
+        return make_kway(32, sc(32 * MiB), device)
+    raise ValueError(name)
+
+
+# ---------------------------------------------------------------------------
+# CPU baseline (oracle/cpu_baseline.c), bounded sample
+# ---------------------------------------------------------------------------
+
+def cpu_baseline(info):
+    """Time the reference's per-rank ring reduce_scatter on host cores for a
+    bounded sample of the workload (same P and dtype, shorter blocks)."""
+    build = os.path.join(ROOT, "oracle", "build")
+    mpi_bin = os.path.join(build, "cpu_baseline_mpi")
+    shm_bin = os.path.join(build, "cpu_baseline_shm")
+    if not os.path.exists(shm_bin):
+        try:
+            subprocess.run(["make", "-C", os.path.join(ROOT, "oracle")], check=True, capture_output=True)
+        except Exception as e:                               # noqa: BLE001
+            return {"value": None, "unit": "GB/s", "cores": 0, "kind": "port", "sample": f"not built: {e}"}
+    P = info["P"] if info["kernel"] in ("k_add_segs", "k_reduce_kway") and info["P"] <= 8 else 8
+    dtype = "bf16" if info["dtype"] == "bf16" else "f32"
+    host_cores = os.cpu_count() or 1
+    ranks = min(P, max(1, host_cores))
+    if ranks & (ranks - 1):
+        ranks = 1 << (ranks.bit_length() - 1)
+    block = (1 << 21) if dtype == "bf16" else (1 << 20)      # 4 MiB blocks
+    args = ["--alg", "ring", "--dtype", dtype, "--block", str(block), "--warmup", "1", "--iters", "5",
+            "--scale", "0.01" if dtype == "bf16" else "1.0"]
+    launcher = None
+    for cand in ("/opt/conda/bin/mpiexec.hydra", shutil.which("mpiexec.hydra"), shutil.which("mpiexec")):
+        if cand and os.path.exists(cand):
+            launcher = cand
+            break
+    attempts = []
+    if launcher and os.path.exists(mpi_bin):
+        attempts.append(([launcher, "-np", str(ranks), mpi_bin] + args, "MPI_Sendrecv (MPICH)"))
+    attempts.append(([shm_bin, "--ranks", str(ranks)] + args, "fork+shared memory"))
+    for cmd, transport in attempts:
+        try:
+            t0 = time.time()
+            p = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+            line = [l for l in p.stdout.splitlines() if l.startswith("{")]
+            if p.returncode == 0 and line:
+                r = json.loads(line[-1])
+                return {"value": round(r["GBps"], 3), "unit": "GB/s", "cores": ranks, "kind": "port",
+                        "ms_per_call": round(r["ms_per_call"], 3), "host_cores": host_cores,
+                        "sample": f"ring reduce_scatter of the reference (pccl/src/reduce_scatter.cpp:101-155) "
+                                  f"on host buffers, {ranks} ranks = {ranks} processes over {transport}, {dtype}, "
+                                  f"{block} elements per block ({ranks * block} per rank), 1 warm-up + 5 timed "
+                                  f"calls, {time.time() - t0:.1f} s wall"}
+        except Exception:                                     # noqa: BLE001
+            continue
+    return {"value": None, "unit": "GB/s", "cores": 0, "kind": "port", "sample": "baseline program failed"}
+
+
+# ---------------------------------------------------------------------------
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs all virtual ranks on ONE GPU and issues no inter-GPU collective; "
+              f"--gpus {args.gpus} is not supported (use --gpus 1).", file=sys.stderr)
+        return 2
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP kernels have no CPU fallback.", file=sys.stderr)
+        return 3
+    from pccl import _native
+    from pccl.build_kernels import build
+    lib = build()
+    for kv in args.tune:
+        k, v = kv.split("=")
+        lib.set_tuning(k, int(v))
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+
+    step, info = build_workload(args.workload, args.mode, args.scale, device)
+    torch.cuda.synchronize()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream()           # the stream the library launches on
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record(stream)
+    for _ in range(args.steps):
+        step()
+    end.record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    dev_ms = start.elapsed_time(end)
+    ms_per_step = dev_ms / args.steps
+    value = info["alg_bytes"] / (ms_per_step * 1e-3) / 1e9
+
+    ok = None
+    if not args.no_verify:
+        ok = bool(info["verify"]())
+
+    # the timed region holds nothing but the dominant kernel's launches (plus, in
+    # faithful mode, the copies), so its mean launch time is region / launches
+    if info["launches"] == info["kernel_launches"]:
+        kernel_ms = dev_ms / (args.steps * info["kernel_launches"])
+    else:
+        kernel_ms = None
+    roof = None
+    if kernel_ms:
+        achieved = info["kernel_bytes"] / (kernel_ms * 1e-3) / 1e9
+        traffic = None
+        tfile = os.path.join(ROOT, "profiles", "traffic.json")
+        if os.path.exists(tfile):
+            try:
+                traffic = json.load(open(tfile)).get(f"{args.workload}:{info['kernel']}")
+            except Exception:                                 # noqa: BLE001
+                traffic = None
+        roof = {"bound": "hbm", "kernel": info["kernel"], "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                "traffic": traffic, "bytes_per_launch": info["kernel_bytes"],
+                "avg_launch_ms": round(kernel_ms, 5)}
+
+    cpu = None if args.no_cpu_baseline else cpu_baseline(info)
+
+    out = {
+        "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": info["dtype"], "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {info['desc']}", "algorithmic_bytes_per_step": info["alg_bytes"],
+                   "launches_per_step": info["launches"], "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
+                   "wall_ms_per_step": round(wall_ms / args.steps, 4), "verified": ok,
+                   "tuning": {k: lib.get_tuning(k) for k in ("grid_cap", "unroll", "nt_load", "nt_store")}},
+        "roofline": roof, "cpu_baseline": cpu,
+    }
+    print(json.dumps(out), flush=True)
+    return 0 if ok in (None, True) else 1
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -371,6 +371,10 @@ __global__ __launch_bounds__(kThreads) void k_gather_multicast(GatherArgs t, int
 #pragma unroll
         for (int j = 0; j < U; ++j) st16<NTS>(dv + base + (size_t)j * kThreads + tid, x[j]);
       }
+      if (tile == 0 && tid < nb - nvec * 16) {   // the last nb % 16 bytes of the shard
+        const size_t i = nvec * 16 + tid;
+        for (int r = 0; r < nout; ++r) ((uint8_t*)t.outs[r])[off + i] = src[i];
+      }
     } else {
       for (int r = 0; r < nout; ++r)
         copy_tile<U, NTL, NTS>((uint8_t*)t.outs[r] + off, src, nb, tile);

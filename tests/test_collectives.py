@@ -1,0 +1,285 @@
+"""GPU parity of whole collectives on virtual ranks against the CPU oracle:
+driver API (all ranks' tensors in one call), every execution mode, and the
+per-rank API run SPMD (one thread per virtual rank) with both backends."""
+import numpy as np
+import pytest
+
+from helpers import (assert_bits_equal, halving_closed_form, make_inputs, ring_closed_form, to_numpy,
+                     to_torch)
+from oracle import pccl_oracle as O
+
+DTYPES = [O.F32, O.BF16]
+MODES = ["steps", "fused", "faithful"]
+
+
+def _tdtype(dtype):
+    import torch
+    return torch.float32 if dtype == O.F32 else torch.bfloat16
+
+
+def _rs_oracle(alg):
+    return O.ring_reduce_scatter if alg == "ring" else O.recursive_halving_reduce_scatter
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("alg,P", [("ring", 1), ("ring", 2), ("ring", 3), ("ring", 4), ("ring", 8), ("ring", 13),
+                                   ("recursive", 1), ("recursive", 2), ("recursive", 4), ("recursive", 8),
+                                   ("recursive", 16), ("recursive", 64)])
+def test_reduce_scatter_driver(target, dtype, mode, alg, P):
+    import torch
+    from pccl import kernels
+    B = 1031 if P <= 16 else 130          # ragged: not a multiple of the vector width
+    print(f"reduce_scatter alg={alg} P={P} B={B} dtype={dtype} mode={mode}", flush=True)
+    ins = make_inputs(P, P * B, dtype, seed=21)
+    t_in = [to_torch(x, dtype, target.device) for x in ins]
+    t_out = [torch.zeros(B, dtype=_tdtype(dtype), device=target.device) for _ in range(P)]
+    kernels.reduce_scatter_ranks(t_out, t_in, algorithm=alg, mode=mode)
+    target.sync()
+    want = _rs_oracle(alg)(ins, dtype)
+    for r in range(P):
+        assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"rank {r}")
+        assert_bits_equal(to_numpy(t_in[r], dtype), ins[r], f"input of rank {r} modified")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_config1_shape_small_ring_p4_uniform(target, dtype):
+    """BASELINE config 1 at reduced length: P=4, uniform[-1,1], seed + rank;
+    all three modes agree with the oracle and with the closed-form left fold."""
+    import torch
+    from pccl import kernels
+    P, B = 4, 1 << 16
+    ins = make_inputs(P, P * B, dtype, seed=1234, dist="uniform")
+    want = O.ring_reduce_scatter(ins, dtype)
+    closed = ring_closed_form(ins, dtype)
+    for r in range(P):
+        assert_bits_equal(want[r], closed[r], "oracle vs closed form")
+    t_in = [to_torch(x, dtype, target.device) for x in ins]
+    for mode in MODES:
+        t_out = [torch.zeros(B, dtype=_tdtype(dtype), device=target.device) for _ in range(P)]
+        kernels.reduce_scatter_ranks(t_out, t_in, "ring", mode)
+        target.sync()
+        for r in range(P):
+            assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"{mode} rank {r}")
+
+
+@pytest.mark.parametrize("alg", ["ring", "recursive"])
+def test_integer_inputs_give_exact_sums(target, alg):
+    """Small integers make every order exact: isolates placement from rounding."""
+    import torch
+    from pccl import kernels
+    P, B = 8, 999
+    for dtype in DTYPES:
+        ins = make_inputs(P, P * B, dtype, seed=3, dist="int")
+        as_f = [x if dtype == O.F32 else O.bf16_to_f32(x) for x in ins]
+        total = np.sum(np.stack(as_f).astype(np.float64), axis=0)
+        t_in = [to_torch(x, dtype, target.device) for x in ins]
+        for mode in MODES:
+            t_out = [torch.zeros(B, dtype=_tdtype(dtype), device=target.device) for _ in range(P)]
+            kernels.reduce_scatter_ranks(t_out, t_in, alg, mode)
+            target.sync()
+            for r in range(P):
+                got = t_out[r].float().cpu().numpy().astype(np.float64)
+                assert np.array_equal(got, total[r * B:(r + 1) * B]), (alg, dtype, mode, r)
+
+
+@pytest.mark.parametrize("mode", ["steps", "fused"])
+@pytest.mark.parametrize("alg,P", [("recursive", 1), ("recursive", 2), ("recursive", 4), ("recursive", 16),
+                                   ("ring", 1), ("ring", 2), ("ring", 3), ("ring", 7), ("ring", 16)])
+@pytest.mark.parametrize("blk", [1, 6, 256, 4096 + 2, 100_000])
+def test_all_gather_driver(target, mode, alg, P, blk):
+    import torch
+    from pccl import kernels
+    print(f"all_gather alg={alg} P={P} blk={blk} mode={mode}", flush=True)
+    rng = np.random.default_rng(5)
+    ins = [rng.integers(0, 256, blk, dtype=np.uint8) for _ in range(P)]
+    t_in = [torch.from_numpy(x).to(target.device) for x in ins]
+    t_out = [torch.full((P * blk,), 0xA5, dtype=torch.uint8, device=target.device) for _ in range(P)]
+    kernels.all_gather_ranks(t_out, t_in, algorithm=alg, mode=mode)
+    target.sync()
+    want = (O.ring_all_gather if alg == "ring" else O.recursive_doubling_all_gather)(ins)
+    cat = torch.cat(t_in)
+    for r in range(P):
+        assert np.array_equal(t_out[r].cpu().numpy(), want[r]), f"rank {r}"
+        assert torch.equal(t_out[r], cat)
+
+
+def test_all_gather_bf16_and_f32_typed(target):
+    import torch
+    from pccl import kernels
+    for td in (torch.bfloat16, torch.float32):
+        P, n = 4, 3001
+        t_in = [torch.randn(n, device=target.device).to(td) for _ in range(P)]
+        t_out = [torch.zeros(P * n, dtype=td, device=target.device) for _ in range(P)]
+        kernels.all_gather_ranks(t_out, t_in, "recursive", "steps")
+        target.sync()
+        for r in range(P):
+            assert torch.equal(t_out[r].view(torch.uint8), torch.cat(t_in).view(torch.uint8))
+
+
+def test_all_gather_uneven_padded_to_256(target):
+    """Uneven ZeRO-style shards, each padded to 256 bytes: equals torch.cat of
+    the unpadded shards at the padded offsets; padding bytes stay untouched."""
+    import torch
+    from pccl import kernels
+    rng = np.random.default_rng(8)
+    P = 16
+    lens = [int(x) for x in rng.integers(1, 40_000, P)]
+    lens[3] = 0
+    lens[5] = 2 * 17          # not a multiple of 4 bytes
+    t_in = [torch.from_numpy(rng.integers(0, 2 ** 15, n, dtype=np.int16)).to(target.device).view(torch.bfloat16)
+            if n else torch.empty(0, dtype=torch.bfloat16, device=target.device) for n in lens]
+
+    def as_bytes(t):
+        return t.view(torch.uint8) if t.numel() else torch.empty(0, dtype=torch.uint8, device=t.device)
+    nbytes = [2 * n for n in lens]
+    off = kernels.padded_offsets(nbytes, 256)
+    total = off[-1] + (nbytes[-1] + 255) // 256 * 256
+    t_out = [torch.full((total,), 0xA5, dtype=torch.uint8, device=target.device) for _ in range(P)]
+    used = kernels.all_gather_uneven_ranks(t_out, t_in, align=256)
+    target.sync()
+    assert used == off and all(o % 256 == 0 for o in off)
+    want = O.uneven_all_gather([as_bytes(t).cpu().numpy() for t in t_in], off, total)
+    for r in range(P):
+        assert np.array_equal(t_out[r].cpu().numpy(), want[r]), f"rank {r}"
+    # closed form: the shards, unpadded, in rank order
+    got = torch.cat([t_out[0][o:o + nb] for o, nb in zip(off, nbytes)])
+    assert torch.equal(got, torch.cat([as_bytes(t) for t in t_in]))
+
+
+# ---------------------------------------------------------------------------
+# per-rank API, SPMD
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("use_rh,P", [(False, 4), (False, 5), (True, 4), (True, 8)])
+@pytest.mark.parametrize("cpp", [True, False])
+def test_reduce_scatter_per_rank_api(target, dtype, use_rh, P, cpp):
+    """_reduce_scatter(out, in, group=comm, ...) called by every virtual rank;
+    the native backend and the Python algorithms give the oracle's bits."""
+    import torch
+    import pccl
+    B = 777
+    print(f"_reduce_scatter P={P} rh={use_rh} cpp={cpp} dtype={dtype}", flush=True)
+    ins = make_inputs(P, P * B, dtype, seed=31)
+    t_in = [to_torch(x, dtype, target.device) for x in ins]
+    t_out = [torch.zeros(B, dtype=_tdtype(dtype), device=target.device) for _ in range(P)]
+    world = pccl.VirtualWorld(P, target.device)
+
+    def rank_main(comm):
+        r = comm.Get_rank()
+        return pccl._reduce_scatter(t_out[r], t_in[r], group=comm, use_rh=use_rh, use_pccl_cpp_backend=cpp)
+
+    assert world.run(rank_main) == [None] * P
+    target.sync()
+    want = _rs_oracle("recursive" if use_rh else "ring")(ins, dtype)
+    for r in range(P):
+        assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"rank {r}")
+
+
+@pytest.mark.parametrize("cpp", [True, False])
+@pytest.mark.parametrize("use_rd", [True, False])
+def test_all_gather_per_rank_api(target, cpp, use_rd):
+    import torch
+    import pccl
+    P, n = 8, 1234
+    t_in = [torch.randn(n, device=target.device).bfloat16() for _ in range(P)]
+    t_out = [torch.zeros(P * n, dtype=torch.bfloat16, device=target.device) for _ in range(P)]
+    world = pccl.VirtualWorld(P, target.device)
+    world.run(lambda comm: pccl._all_gather(t_out[comm.Get_rank()], t_in[comm.Get_rank()], group=comm,
+                                            use_rd=use_rd, use_pccl_cpp_backend=cpp))
+    target.sync()
+    for r in range(P):
+        assert torch.equal(t_out[r].view(torch.int16), torch.cat(t_in).view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("intra,inter", [(2, 2), (4, 2), (2, 4)])
+@pytest.mark.parametrize("use_rh", [True, False])
+@pytest.mark.parametrize("cpp", [True, False])
+def test_reduce_scatter_2D(target, dtype, intra, inter, use_rh, cpp):
+    import torch
+    import pccl
+    world_size = intra * inter
+    m = 333
+    print(f"reduce_scatter_2D {intra}x{inter} rh={use_rh} cpp={cpp} dtype={dtype}", flush=True)
+    ins = make_inputs(world_size, world_size * m, dtype, seed=41)
+    t_in = [to_torch(x, dtype, target.device) for x in ins]
+    t_out = [torch.zeros(m, dtype=_tdtype(dtype), device=target.device) for _ in range(world_size)]
+    world = pccl.VirtualWorld(world_size, target.device)
+
+    def rank_main(comm):
+        r = comm.Get_rank()
+        pg = pccl.ProcessGroups(intra, inter, inner_group_backend="mpi", outer_group_backend="mpi", comm=comm)
+        assert pg.get_world_size() == [intra, inter]
+        pccl.reduce_scatter_2D(t_out[r], t_in[r], group=pg, use_rh=use_rh, use_pccl_cpp_backend=cpp)
+
+    world.run(rank_main)
+    target.sync()
+    want = O.reduce_scatter_2d(ins, intra, inter, dtype, "recursive" if use_rh else "ring")
+    for r in range(world_size):
+        assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"rank {r}")
+
+
+@pytest.mark.parametrize("intra,inter", [(2, 2), (4, 2), (2, 4)])
+@pytest.mark.parametrize("use_rd", [True, False])
+@pytest.mark.parametrize("cpp", [True, False])
+def test_all_gather_2D(target, intra, inter, use_rd, cpp):
+    import torch
+    import pccl
+    world_size = intra * inter
+    n = 501
+    t_in = [torch.randn(n, device=target.device) for _ in range(world_size)]
+    t_out = [torch.zeros(world_size * n, device=target.device) for _ in range(world_size)]
+    world = pccl.VirtualWorld(world_size, target.device)
+
+    def rank_main(comm):
+        r = comm.Get_rank()
+        pg = pccl.ProcessGroups(intra, inter, comm=comm)
+        pccl.all_gather_2D(t_out[r], t_in[r], group=pg, use_rd=use_rd, use_pccl_cpp_backend=cpp)
+
+    world.run(rank_main)
+    target.sync()
+    want = O.all_gather_2d([t.cpu().numpy() for t in t_in], intra, inter, "recursive" if use_rd else "ring")
+    cat = torch.cat(t_in)
+    for r in range(world_size):
+        assert np.array_equal(t_out[r].view(torch.uint8).cpu().numpy(), want[r]), f"rank {r}"
+        assert torch.equal(t_out[r], cat)      # the 2-D all_gather is a plain concatenation
+
+
+@pytest.mark.parametrize("rec", [True, False])
+def test_all_reduce(target, rec):
+    import torch
+    import pccl
+    P, n = 4, 4 * 257
+    dtype = O.F32
+    ins = make_inputs(P, n, dtype, seed=51)
+    t = [to_torch(x, dtype, target.device) for x in ins]
+    world = pccl.VirtualWorld(P, target.device)
+    world.run(lambda comm: pccl._all_reduce(t[comm.Get_rank()], group=comm, use_rh_and_rd=rec))
+    target.sync()
+    want = O.all_reduce(ins, dtype, "recursive" if rec else "ring")
+    for r in range(P):
+        assert_bits_equal(to_numpy(t[r], dtype), want[r], f"rank {r}")
+
+
+def test_request_wait_runs_epilogue(target):
+    import torch
+    import pccl
+    if target.device == "cpu":
+        pytest.skip("a StreamRequest records a HIP event")
+    P, n = 2, 64
+    t_in = [torch.randn(n, device=target.device) for _ in range(P)]
+    t_out = [torch.zeros(P * n, device=target.device) for _ in range(P)]
+    world = pccl.VirtualWorld(P, target.device)
+    called = []
+
+    def rank_main(comm):
+        r = comm.Get_rank()
+        req = pccl._all_gather(t_out[r], t_in[r], group=comm, async_op=True)
+        assert isinstance(req, pccl.Request)
+        req.wait(lambda: called.append(r))
+
+    world.run(rank_main)
+    assert sorted(called) == [0, 1]
+    assert torch.equal(t_out[0], torch.cat(t_in))

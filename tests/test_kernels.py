@@ -1,0 +1,240 @@
+"""GPU parity of the individual HIP kernels against the CPU oracle, through the
+C ABI (ctypes -> libpccl_hip.so).  Bit-exact: these are IEEE adds in a fixed
+order and byte copies."""
+import numpy as np
+import pytest
+
+from helpers import assert_bits_equal, make_inputs, to_numpy, to_torch
+from oracle import pccl_oracle as O
+
+DTYPES = [O.F32, O.BF16]
+CODE = {O.F32: 0, O.BF16: 1}
+
+
+# sizes: empty, sub-vector, one vector, ragged, exactly one tile (256*4 vectors), several tiles + tail
+SIZES = [0, 1, 3, 4, 8, 9, 255, 1024, 4096, 4097, 8192 + 5, 300_001]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n", SIZES)
+def test_accumulate_matches_oracle(target, dtype, n):
+    import torch
+    print(f"accumulate dtype={dtype} n={n}", flush=True)
+    a, b = make_inputs(2, n, dtype, seed=11)
+    ta, tb = to_torch(a, dtype, target.device), to_torch(b, dtype, target.device)
+    target.native.accumulate(ta.data_ptr(), tb.data_ptr(), n, CODE[dtype], target.stream())
+    target.sync()
+    assert_bits_equal(to_numpy(ta, dtype), O.vector_add(a, b, dtype), "accumulate")
+    assert_bits_equal(to_numpy(tb, dtype), b, "src untouched")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shift", [(0, 0, 0), (1, 1, 1), (3, 3, 3), (1, 2, 3), (0, 1, 0)])
+def test_add_any_alignment(target, dtype, shift):
+    """Operands that start off a 16-byte boundary: common misalignment takes the
+    peeled vector path, different misalignments the element path."""
+    import torch
+    n = 5000
+    print(f"add alignment dtype={dtype} shift={shift}", flush=True)
+    a, b = make_inputs(2, n + 8, dtype, seed=5)
+    ta, tb = to_torch(a, dtype, target.device), to_torch(b, dtype, target.device)
+    td = torch.zeros(n + 16, dtype=ta.dtype, device=target.device)
+    sd, sa, sb = shift
+    es = ta.element_size()
+    target.native.add(td.data_ptr() + sd * es, ta.data_ptr() + sa * es, tb.data_ptr() + sb * es, n, CODE[dtype],
+               target.stream())
+    target.sync()
+    got = to_numpy(td, dtype)
+    assert_bits_equal(got[sd:sd + n], O.vector_add(a[sa:sa + n], b[sb:sb + n], dtype), "add")
+    assert not got[:sd].any() and not got[sd + n:].any(), "wrote outside the destination"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_bf16_and_f32_special_values(target, dtype):
+    """Infinities, NaN, signed zeros, denormals and rounding ties go through the
+    same bits as the oracle."""
+    import torch
+    if dtype == O.F32:
+        vals = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 3.4e38, 1e-38,
+                         1.0 + 2 ** -23, 2 ** -24, 16777216.0], dtype=np.float32)
+    else:
+        # every bf16 exponent with a few mantissas, plus specials
+        pats = [0x0000, 0x8000, 0x3F80, 0xBF80, 0x7F80, 0xFF80, 0x7FC0, 0x0001, 0x8001, 0x7F7F, 0x0080,
+                0x3F81, 0x3B80, 0x4B80, 0x3FFF, 0x4000, 0x3C00, 0x3C01]
+        vals = np.array(pats, dtype=np.uint16)
+    a = np.repeat(vals, vals.size)
+    b = np.tile(vals, vals.size)
+    ta, tb = to_torch(a, dtype, target.device), to_torch(b, dtype, target.device)
+    target.native.accumulate(ta.data_ptr(), tb.data_ptr(), a.size, CODE[dtype], target.stream())
+    target.sync()
+    assert_bits_equal(to_numpy(ta, dtype), O.vector_add(a, b, dtype), "special values")
+
+
+def test_bf16_add_all_exponent_pairs(target):
+    """All 2^16 bf16 patterns against 64 partners spanning the exponent range."""
+    import torch
+    a = np.arange(65536, dtype=np.uint16)
+    partners = np.concatenate([np.arange(0, 65536, 2048, dtype=np.uint16) | np.uint16(0x55),
+                               np.arange(0, 65536, 2048, dtype=np.uint16) | np.uint16(0x2A)])
+    A = np.tile(a, partners.size)
+    Bv = np.repeat(partners, a.size)
+    ta, tb = to_torch(A, O.BF16, target.device), to_torch(Bv, O.BF16, target.device)
+    target.native.accumulate(ta.data_ptr(), tb.data_ptr(), A.size, 1, target.stream())
+    target.sync()
+    assert_bits_equal(to_numpy(ta, O.BF16), O.vector_add(A, Bv, O.BF16), "bf16 exhaustive")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("count,n", [(1, 1000), (5, 4099), (64, 777)])
+def test_add_batched(target, dtype, count, n):
+    import torch
+    print(f"add_batched dtype={dtype} count={count} n={n}", flush=True)
+    a = make_inputs(count, n, dtype, seed=1)
+    b = make_inputs(count, n, dtype, seed=100)
+    ta = [to_torch(x, dtype, target.device) for x in a]
+    tb = [to_torch(x, dtype, target.device) for x in b]
+    td = [torch.zeros_like(t) for t in ta]
+    target.native.add_batched([t.data_ptr() for t in td], [t.data_ptr() for t in ta], [t.data_ptr() for t in tb],
+                       n, CODE[dtype], target.stream())
+    target.sync()
+    for s in range(count):
+        assert_bits_equal(to_numpy(td[s], dtype), O.vector_add(a[s], b[s], dtype), f"segment {s}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("k", [2, 3, 4, 7, 8, 16, 32, 64])
+@pytest.mark.parametrize("order", ["ring", "halving"])
+def test_reduce_kway_matches_sequential_hops(target, dtype, k, order):
+    """The fused reduce equals k-1 oracle hops in the schedule's order."""
+    import torch
+    if order == "halving" and k & (k - 1):
+        pytest.skip("halving order needs a power of two")
+    n = 3001
+    first = (k // 3) % k
+    print(f"reduce_kway dtype={dtype} k={k} order={order} first={first}", flush=True)
+    shards = make_inputs(k, n, dtype, seed=7)
+    ts = [to_torch(x, dtype, target.device) for x in shards]
+    out = torch.zeros_like(ts[0])
+    target.native.reduce_kway(out.data_ptr(), [t.data_ptr() for t in ts], n, CODE[dtype],
+                       0 if order == "ring" else 1, first, True, target.stream())
+    target.sync()
+    if order == "ring":
+        want = shards[first]
+        for t in range(1, k):
+            want = O.vector_add(want, shards[(first + t) % k], dtype)
+    else:
+        v = [shards[first ^ m] for m in range(k)]
+        h = k // 2
+        while h >= 1:
+            for m in range(h):
+                v[m] = O.vector_add(v[m], v[m + h], dtype)
+            h //= 2
+        want = v[0]
+    assert_bits_equal(to_numpy(out, dtype), want, "reduce_kway")
+
+
+def test_reduce_kway_bf16_single_rounding(target):
+    """per_hop_round=0: fp32 partial sums, one rounding at the end (within 1 ulp
+    of the per-hop result per hop; here checked exactly against numpy)."""
+    import torch
+    k, n = 8, 4099
+    shards = make_inputs(k, n, O.BF16, seed=3)
+    ts = [to_torch(x, O.BF16, target.device) for x in shards]
+    out = torch.zeros_like(ts[0])
+    target.native.reduce_kway(out.data_ptr(), [t.data_ptr() for t in ts], n, 1, 0, 0, False,
+                       target.stream())
+    target.sync()
+    acc = O.bf16_to_f32(shards[0])
+    for t in range(1, k):
+        acc = (acc + O.bf16_to_f32(shards[t])).astype(np.float32)
+    assert_bits_equal(to_numpy(out, O.BF16), O.f32_to_bf16(acc), "single rounding")
+
+
+@pytest.mark.parametrize("sizes", [[0], [1], [15, 16, 17], [4096, 1, 70000, 0, 33], [5] * 64])
+@pytest.mark.parametrize("shift", [0, 1, 4])
+def test_copy_batched_ragged(target, sizes, shift):
+    import torch
+    print(f"copy_batched sizes={sizes[:5]} shift={shift}", flush=True)
+    rng = np.random.default_rng(0)
+    srcs = [rng.integers(0, 256, s + 8, dtype=np.uint8) for s in sizes]
+    ts = [torch.from_numpy(x).to(target.device) for x in srcs]
+    td = [torch.full((s + 32,), 0xA5, dtype=torch.uint8, device=target.device) for s in sizes]
+    target.native.copy_batched([t.data_ptr() + 16 + shift for t in td], [t.data_ptr() + shift for t in ts], sizes,
+                        target.stream())
+    target.sync()
+    for s, src, dst in zip(sizes, srcs, td):
+        got = dst.cpu().numpy()
+        assert np.array_equal(got[16 + shift:16 + shift + s], src[shift:shift + s])
+        assert (got[:16 + shift] == 0xA5).all() and (got[16 + shift + s:] == 0xA5).all()
+
+
+def test_copy_mismatched_alignment(target):
+    import torch
+    rng = np.random.default_rng(1)
+    src = rng.integers(0, 256, 10007, dtype=np.uint8)
+    ts = torch.from_numpy(src).to(target.device)
+    for ds, ss in [(1, 2), (4, 8), (3, 0), (0, 5)]:
+        n = 9990
+        td = torch.full((n + 32,), 0x5A, dtype=torch.uint8, device=target.device)
+        target.native.copy_batched([td.data_ptr() + ds], [ts.data_ptr() + ss], [n], target.stream())
+        target.sync()
+        got = td.cpu().numpy()
+        assert np.array_equal(got[ds:ds + n], src[ss:ss + n]), (ds, ss)
+        assert (got[:ds] == 0x5A).all() and (got[ds + n:] == 0x5A).all()
+
+
+@pytest.mark.parametrize("rows,cols,m", [(2, 4, 64), (4, 2, 6), (8, 8, 4096 + 16), (1, 5, 3), (3, 1, 10)])
+def test_block_transpose(target, rows, cols, m):
+    import torch
+    x = np.random.default_rng(2).integers(0, 256, rows * cols * m, dtype=np.uint8)
+    tx = torch.from_numpy(x).to(target.device)
+    ty = torch.zeros_like(tx)
+    target.native.block_transpose(ty.data_ptr(), tx.data_ptr(), rows, cols, m, target.stream())
+    target.sync()
+    assert np.array_equal(ty.cpu().numpy(), O.block_transpose(x, rows, cols))
+    want = tx.view(rows, cols, -1).transpose(0, 1).reshape(-1)
+    assert torch.equal(ty, want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("P", [2, 4, 8])
+def test_rh_round_is_the_pairwise_half_add(target, dtype, P):
+    """One round in place on the work buffers against the two branches of the
+    reference written out with numpy slices."""
+    import torch
+    B = 517
+    bufs = make_inputs(P, P * B, dtype, seed=9)
+    tb = [to_torch(x, dtype, target.device) for x in bufs]
+    cur = [x.copy() for x in bufs]
+    rounds = P.bit_length() - 1
+    for rnd in range(rounds):
+        target.native.rh_round([t.data_ptr() for t in tb], None, None, P, B, rnd, CODE[dtype],
+                        target.stream())
+        target.sync()
+        group = P >> rnd
+        half = group // 2
+        count = half * B
+        snap = [c.copy() for c in cur]
+        for r in range(P):
+            start = (r // group) * group * B
+            if r % group < half:
+                p = r + half
+                cur[r][start:start + count] = O.vector_add(snap[r][start:start + count],
+                                                           snap[p][start:start + count], dtype)
+            else:
+                p = r - half
+                cur[r][start + count:start + 2 * count] = O.vector_add(
+                    snap[r][start + count:start + 2 * count], snap[p][start + count:start + 2 * count], dtype)
+        for r in range(P):
+            assert_bits_equal(to_numpy(tb[r], dtype), cur[r], f"round {rnd} rank {r}")
+
+
+def test_invalid_arguments_return_codes(target):
+    """Errors come back as codes + messages; nothing is launched."""
+    from pccl._native import NativeError
+    with pytest.raises(NativeError, match="unknown dtype"):
+        target.native.accumulate(16, 16, 4, 7)
+    with pytest.raises(NativeError, match="Unknown algorithm specified for reduce_scatter_mpi: tree"):
+        target.native.reduce_scatter_virtual([16], [16], None, 4, 0, "tree")
+    with pytest.raises(NativeError, match="power-of-two"):
+        target.native.reduce_scatter_virtual([16] * 3, [16] * 3, [16] * 3, 4, 0, "recursive")
