@@ -55,6 +55,9 @@ def parse_args():
                     help="shrink the per-rank message by this factor (1.0 = BASELINE size)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="after the timed region launch one plain 1 GiB device copy (k_copy_segs): its "
+                         "FETCH_SIZE / WRITE_SIZE readings scale the hardware counters of a rocprofv3 --pmc run")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="launch tuning of the library (grid_cap, unroll, nt_load, nt_store)")
     return ap.parse_args()
@@ -349,6 +352,15 @@ def main():
     dev_ms = start.elapsed_time(end)
     ms_per_step = dev_ms / args.steps
     value = info["alg_bytes"] / (ms_per_step * 1e-3) / 1e9
+
+    if args.calibrate_copy:
+        from pccl import kernels
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=device).fill_(7)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        kernels.copy(dst, src)            # exactly 1 GiB read + 1 GiB written
+        torch.cuda.synchronize()
+        del src, dst
 
     ok = None
     if not args.no_verify:

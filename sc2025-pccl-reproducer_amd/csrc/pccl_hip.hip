@@ -47,8 +47,8 @@ int launch_status(const char* what) {
 
 std::atomic<long> g_grid_cap{0};
 std::atomic<long> g_unroll{4};
-std::atomic<long> g_nt_load{0};
-std::atomic<long> g_nt_store{0};
+std::atomic<long> g_nt_load{1};
+std::atomic<long> g_nt_store{1};
 
 }  // namespace
 
