@@ -75,7 +75,8 @@ def vector_add(a: np.ndarray, b: np.ndarray, dtype: str) -> np.ndarray:
     f32: one IEEE-754 binary32 RNE add (pccl/src/common.cu:8).
     bf16: RNE_bf16(float(a) + float(b)), the fp32 sum itself RNE."""
     if dtype == F32:
-        return (np.asarray(a, np.float32) + np.asarray(b, np.float32)).astype(np.float32)
+        with np.errstate(over="ignore", invalid="ignore"):
+            return (np.asarray(a, np.float32) + np.asarray(b, np.float32)).astype(np.float32)
     if dtype == BF16:
         with np.errstate(over="ignore", invalid="ignore"):
             s = bf16_to_f32(a) + bf16_to_f32(b)

@@ -101,12 +101,8 @@ class Target:
         return torch.cuda.current_stream().cuda_stream
 
 
-@pytest.fixture(params=[pytest.param("hip", marks=pytest.mark.gpu), "cpu-build"])
-def target(request, monkeypatch):
+def _cpu_target(monkeypatch):
     from pccl import _native, kernels
-    if request.param == "hip":
-        # the product library: must already be in the tree; missing = error, not skip
-        return Target("hip", "cuda:0", _native.load())
     lib = _native.NativeLib(build_cpu_library())
 
     def check_host_tensor(t, name):
@@ -117,3 +113,20 @@ def target(request, monkeypatch):
     monkeypatch.setattr(kernels, "check_device_tensor", check_host_tensor)
     monkeypatch.setattr(kernels, "stream_handle", lambda: 0)
     return Target("cpu-build", "cpu", lib)
+
+
+@pytest.fixture(params=[pytest.param("hip", marks=pytest.mark.gpu), "cpu-build"])
+def target(request, monkeypatch):
+    """Parity tests run twice: on the GPU through libpccl_hip.so (marked gpu),
+    and on the CPU build of the same source (indexing and schedules)."""
+    if request.param == "hip":
+        from pccl import _native
+        # the product library: must already be in the tree; missing = error, not skip
+        return Target("hip", "cuda:0", _native.load())
+    return _cpu_target(monkeypatch)
+
+
+@pytest.fixture
+def cpu(monkeypatch):
+    """The CPU build only (host-logic tests)."""
+    return _cpu_target(monkeypatch)

@@ -1,0 +1,71 @@
+#!/usr/bin/env python3
+"""Writes the golden vectors in this folder from the CPU oracle.
+
+The reference ships no fixtures (its only check is an allclose against NCCL on
+unseeded inputs, benchmark_raw_collectives/utils.py:35-42), so these vectors
+come from this repository's oracle (oracle/pccl_oracle.py), whose schedules
+are pinned independently by the closed forms in tests/test_oracle.py.  Each
+.npz holds the inputs of every rank and the expected output of every rank:
+    in_<r>   rank r's input   (float32, or uint16 bfloat16 bit patterns)
+    out_<r>  rank r's output
+    meta     JSON: collective, algorithm, dtype, P, block elements
+Run:  python tests/golden/make_golden.py   (rewrites the files in place)
+"""
+import json
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+from oracle import pccl_oracle as O  # noqa: E402
+
+
+def inputs(P, n, dtype, seed, kind):
+    xs = []
+    for r in range(P):
+        rng = np.random.default_rng(seed + r)
+        if kind == "uniform":                      # BASELINE config 1: uniform[-1, 1], seed + rank
+            x = (rng.random(n, dtype=np.float32) * 2 - 1)
+        elif kind == "grad":                       # BASELINE config 2: normal(0, 1e-2)
+            x = rng.standard_normal(n, dtype=np.float32) * np.float32(1e-2)
+        else:                                      # normal(0, 1)
+            x = rng.standard_normal(n, dtype=np.float32)
+        xs.append(x if dtype == O.F32 else O.f32_to_bf16(x))
+    return xs
+
+
+CASES = [
+    # name, collective, algorithm, dtype, P, B, input kind
+    ("rs_ring_p4_f32_uniform", "reduce_scatter", "ring", O.F32, 4, 48, "uniform"),
+    ("rs_ring_p8_bf16_grad", "reduce_scatter", "ring", O.BF16, 8, 40, "grad"),
+    ("rs_ring_p3_bf16", "reduce_scatter", "ring", O.BF16, 3, 19, "normal"),
+    ("rs_halving_p8_bf16", "reduce_scatter", "recursive", O.BF16, 8, 24, "normal"),
+    ("rs_halving_p4_f32", "reduce_scatter", "recursive", O.F32, 4, 33, "normal"),
+    ("rs_halving_p2_f32", "reduce_scatter", "recursive", O.F32, 2, 64, "uniform"),
+    ("ag_doubling_p8_bf16", "all_gather", "recursive", O.BF16, 8, 21, "normal"),
+    ("ag_ring_p5_f32", "all_gather", "ring", O.F32, 5, 7, "normal"),
+]
+
+
+def main():
+    for name, coll, alg, dtype, P, B, kind in CASES:
+        if coll == "reduce_scatter":
+            xs = inputs(P, P * B, dtype, 1234, kind)
+            fn = O.ring_reduce_scatter if alg == "ring" else O.recursive_halving_reduce_scatter
+            outs = fn(xs, dtype)
+        else:
+            xs = inputs(P, B, dtype, 1234, kind)
+            fn = O.ring_all_gather if alg == "ring" else O.recursive_doubling_all_gather
+            outs = [o.view(xs[0].dtype) for o in fn(xs)]
+        arrays = {f"in_{r}": xs[r] for r in range(P)}
+        arrays.update({f"out_{r}": outs[r] for r in range(P)})
+        meta = dict(collective=coll, algorithm=alg, dtype=dtype, P=P, B=B, inputs=kind)
+        arrays["meta"] = np.frombuffer(json.dumps(meta).encode(), dtype=np.uint8)
+        np.savez(os.path.join(HERE, name + ".npz"), **arrays)
+        print("wrote", name)
+
+
+if __name__ == "__main__":
+    main()

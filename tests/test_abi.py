@@ -1,0 +1,118 @@
+"""The C-ABI library loads without a GPU, exports every symbol the header
+declares, and rejects bad arguments with a code and a message before anything
+is launched.  No compute call is made here."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "pccl_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pccl_hip_\w+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    syms = declared_symbols()
+    for must in ("pccl_hip_accumulate", "pccl_hip_add_batched", "pccl_hip_rh_round", "pccl_hip_reduce_kway",
+                 "pccl_hip_copy_batched", "pccl_hip_gather_place", "pccl_hip_reduce_scatter_virtual",
+                 "pccl_hip_all_gather_virtual", "pccl_hip_last_error", "pccl_hip_version"):
+        assert must in syms
+
+
+def test_library_exports_every_declared_symbol():
+    from pccl import _native
+    assert os.path.exists(_native.LIB_PATH), "libpccl_hip.so has not been built (make -C sc2025-pccl-reproducer_amd/csrc)"
+    lib = ctypes.CDLL(_native.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(lib, name), f"{name} declared in pccl_hip.h but not exported"
+    # and the Python binding knows every one of them
+    assert sorted(_native.SIGNATURES) == declared_symbols()
+
+
+def test_header_compiles_as_plain_c():
+    src = '#include "pccl_hip.h"\nint main(void){return PCCL_HIP_MAX_RANKS == 64 ? 0 : 1;}\n'
+    p = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),
+                        "-x", "c", "-", "-o", "/dev/null"], input=src, text=True, capture_output=True)
+    assert p.returncode == 0, p.stderr
+
+
+def test_version_and_dtype_sizes():
+    from pccl import _native
+    lib = _native.load()
+    assert lib.version() == _native.ABI_VERSION == 1
+    assert lib.dtype_size(_native.F32) == 4 and lib.dtype_size(_native.BF16) == 2 and lib.dtype_size(9) == 0
+
+
+def test_argument_errors_are_codes_with_messages():
+    """Validation happens on the host before any launch, so this runs without a GPU."""
+    from pccl import _native
+    lib = _native.load()
+    E = _native.NativeError
+    with pytest.raises(E, match="unknown dtype"):
+        lib.accumulate(64, 64, 8, 5)
+    with pytest.raises(E, match="NULL operand"):
+        lib.add(0, 64, 64, 8, 0)
+    with pytest.raises(E, match=r"count 65 outside"):
+        lib.add_batched([64] * 65, [64] * 65, [64] * 65, 8, 0)
+    with pytest.raises(E, match=r"a\[1\] is NULL"):
+        lib.add_batched([64, 64], [64, 0], [64, 64], 8, 0)
+    with pytest.raises(E, match="power of two"):
+        lib.rh_round([64] * 3, None, None, 3, 8, 0, 0)
+    with pytest.raises(E, match="round 2 outside"):
+        lib.rh_round([64] * 4, None, None, 4, 8, 2, 0)
+    with pytest.raises(E, match="k = 1 outside"):
+        lib.reduce_kway(64, [64], 8, 0)
+    with pytest.raises(E, match="halving order needs"):
+        lib.reduce_kway(64, [64] * 3, 8, 0, _native.ORDER_HALVING)
+    with pytest.raises(E, match="first = 4 outside"):
+        lib.reduce_kway(64, [64] * 4, 8, 0, _native.ORDER_RING, 4)
+    # the reference's wording for an unknown algorithm (pccl/src/pccl.cpp:83,140)
+    with pytest.raises(E, match="Unknown algorithm specified for reduce_scatter_mpi: tree"):
+        lib.reduce_scatter_virtual([64], [64], None, 8, 0, "tree")
+    with pytest.raises(E, match="Unknown algorithm specified for all_gather_mpi: tree"):
+        lib.all_gather_virtual([64], [64], 8, "tree")
+    with pytest.raises(E, match="power-of-two"):
+        lib.reduce_scatter_virtual([64] * 6, [64] * 6, [64] * 6, 8, 0, "recursive")
+    with pytest.raises(E, match="work is NULL"):
+        lib.reduce_scatter_virtual([64] * 4, [64] * 4, None, 8, 0, "ring", _native.MODE_STEPS)
+    with pytest.raises(E, match="P = 65 outside"):
+        lib.all_gather_virtual([64] * 65, [64] * 65, 8, "ring")
+    with pytest.raises(E, match="unknown key"):
+        lib.set_tuning("bogus", 1)
+    with pytest.raises(E, match="unroll must be"):
+        lib.set_tuning("unroll", 3)
+    assert "unroll must be" in lib.last_error()
+
+
+def test_empty_work_is_accepted_without_a_launch():
+    from pccl import _native
+    lib = _native.load()
+    lib.accumulate(0, 0, 0, 0)
+    lib.add_batched([], [], [], 8, 0)
+    lib.copy_batched([64], [64], [0])
+    lib.reduce_scatter_virtual([64] * 2, [64] * 2, None, 0, 0, "ring")
+    lib.all_gather_virtual([64] * 2, [64] * 2, 0, "recursive")
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    from pccl import _native
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _native.NativeLib(str(tmp_path / "libpccl_hip.so"))
+
+
+def test_cpu_tensors_are_rejected():
+    """The product path never computes on the CPU."""
+    import torch
+    from pccl import kernels
+    a = torch.zeros(8)
+    with pytest.raises(RuntimeError, match="must reside on the GPU"):
+        kernels.accumulate(a, a.clone())
+    with pytest.raises(RuntimeError, match="must reside on the GPU"):
+        kernels.reduce_scatter_ranks([torch.zeros(4)] * 2, [torch.zeros(8)] * 2, "ring")

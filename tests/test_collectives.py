@@ -147,6 +147,35 @@ def test_all_gather_uneven_padded_to_256(target):
     assert torch.equal(got, torch.cat([as_bytes(t) for t in t_in]))
 
 
+def _golden_cases():
+    import glob
+    import os
+    here = os.path.dirname(os.path.abspath(__file__))
+    return sorted(glob.glob(os.path.join(here, "golden", "*.npz")))
+
+
+@pytest.mark.parametrize("path", _golden_cases(), ids=lambda p: p.split("/")[-1][:-4])
+@pytest.mark.parametrize("mode", MODES)
+def test_golden_vectors(target, path, mode):
+    """The committed fixtures (tests/golden/make_golden.py) through the library."""
+    import json
+    import torch
+    from pccl import kernels
+    z = np.load(path)
+    meta = json.loads(bytes(z["meta"]).decode())
+    P, dtype = meta["P"], meta["dtype"]
+    t_in = [to_torch(z[f"in_{r}"], dtype, target.device) for r in range(P)]
+    if meta["collective"] == "reduce_scatter":
+        t_out = [torch.zeros(meta["B"], dtype=_tdtype(dtype), device=target.device) for _ in range(P)]
+        kernels.reduce_scatter_ranks(t_out, t_in, meta["algorithm"], mode)
+    else:
+        t_out = [torch.zeros(P * meta["B"], dtype=_tdtype(dtype), device=target.device) for _ in range(P)]
+        kernels.all_gather_ranks(t_out, t_in, meta["algorithm"], mode)
+    target.sync()
+    for r in range(P):
+        assert_bits_equal(to_numpy(t_out[r], dtype), z[f"out_{r}"], f"rank {r}")
+
+
 # ---------------------------------------------------------------------------
 # per-rank API, SPMD
 # ---------------------------------------------------------------------------
