@@ -42,6 +42,20 @@ __device__ __forceinline__ uint32_t bf16_round_hi(float s) {
   return (s != s) ? 0x7fc00000u : r;
 }
 
+// Two fp32 values to packed bfloat16 (lo in bits 0-15) with the gfx950 packed
+// conversion: round to nearest even, identical to bf16_round_hi for every
+// non-NaN input; a NaN stays a (quiet) NaN but keeps its payload, so results
+// that may be NaN are canonicalised with bf16_round_hi when they are stored.
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
+  f32x2 v = {lo, hi};
+  bf16x2 r = __builtin_convertvector(v, bf16x2);
+  uint32_t u;
+  __builtin_memcpy(&u, &r, 4);
+  return u;
+}
+
 struct OpF32 {
   typedef float elem;
   static constexpr int kPerVec = 4;
@@ -90,6 +104,11 @@ struct AccF32 {
     f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
   }
   static __device__ __forceinline__ float hop(float a, float b) { return a + b; }
+  template <int L>
+  static __device__ __forceinline__ void hop_lanes(float* acc, const float* x) {
+#pragma unroll
+    for (int l = 0; l < L; ++l) acc[l] = acc[l] + x[l];
+  }
   static __device__ __forceinline__ u32x4 narrow(const float* f) {
     u32x4 r;
     r.x = __float_as_uint(f[0]); r.y = __float_as_uint(f[1]);
@@ -112,6 +131,22 @@ struct AccBF16 {
     float s = a + b;
     if constexpr (PER_HOP) return __uint_as_float(bf16_round_hi(s));
     else return s;
+  }
+  // acc[l] = hop(acc[l], x[l]) for L lanes; lanes are rounded two at a time
+  // with the packed conversion (NaN payloads are settled in narrow()).
+  template <int L>
+  static __device__ __forceinline__ void hop_lanes(float* acc, const float* x) {
+    if constexpr (PER_HOP && (L % 2 == 0)) {
+#pragma unroll
+      for (int l = 0; l < L; l += 2) {
+        const uint32_t p = cvt_pk_bf16(acc[l] + x[l], acc[l + 1] + x[l + 1]);
+        acc[l] = __uint_as_float(p << 16);
+        acc[l + 1] = __uint_as_float(p & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int l = 0; l < L; ++l) acc[l] = hop(acc[l], x[l]);
+    }
   }
   static __device__ __forceinline__ u32x4 narrow(const float* f) {
     u32x4 r;
@@ -413,14 +448,15 @@ __device__ __forceinline__ void tree_sum(Load& load, int first, float* out) {
     float lo[L], hi[L];
     tree_sum<Acc, K, M, 2 * H, L>(load, first, lo);
     tree_sum<Acc, K, M + H, 2 * H, L>(load, first, hi);
+    Acc::template hop_lanes<L>(lo, hi);
 #pragma unroll
-    for (int l = 0; l < L; ++l) out[l] = Acc::hop(lo[l], hi[l]);
+    for (int l = 0; l < L; ++l) out[l] = lo[l];
   }
 }
 
 // Fold the k shards at one position in the order of a schedule.
 //   K == 0 : ring order, runtime k: first, first+1, ... (mod k), loads issued
-//            in batches of four ahead of the adds
+//            in batches of eight ahead of the adds
 //   K >= 2 : halving order for k == K: leaves v[m] = shard[first ^ m] summed by
 //            the butterfly v[m] += v[m+h], h = K/2 .. 1, evaluated depth first
 //            by tree_sum (the same tree with only log2 K live partial sums).
@@ -431,24 +467,21 @@ __device__ __forceinline__ void fold_shards(Load&& load, int k, int first, float
     int q = first;
     load(q, acc);
     int done = 1;
-    for (; done + 4 <= k; done += 4) {
-      float f[4][L];
+    for (; done + 8 <= k; done += 8) {
+      float f[8][L];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < 8; ++i) {
         q = q + 1 == k ? 0 : q + 1;
         load(q, f[i]);
       }
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int l = 0; l < L; ++l) acc[l] = Acc::hop(acc[l], f[i][l]);
+      for (int i = 0; i < 8; ++i) Acc::template hop_lanes<L>(acc, f[i]);
     }
     for (; done < k; ++done) {
       q = q + 1 == k ? 0 : q + 1;
       float f[L];
       load(q, f);
-#pragma unroll
-      for (int l = 0; l < L; ++l) acc[l] = Acc::hop(acc[l], f[l]);
+      Acc::template hop_lanes<L>(acc, f);
     }
   } else {
     tree_sum<Acc, K, 0, 1, L>(load, first, acc);
