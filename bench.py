@@ -18,6 +18,8 @@ Workloads (BASELINE.json `configs`; `cfg2` is the one the metric is quoted on):
   cfg4  all_gather placement, P=16, bf16 shards of 128 MiB into 2 GiB outputs
   cfg4u the same with uneven shards padded to 256 bytes
   cfg5  fused one-pass reduce of 32 fp32 shards of 32 Mi elements
+  latency  small messages, 4 KiB .. 1 MiB in bf16: microseconds per accumulate,
+        per copy and per whole P=8 ring reduce_scatter (per-step and fused)
 
 The CPU baseline (the reference's per-rank algorithm on host cores, one process
 per rank over MPI_Sendrecv, or fork+shared memory where no MPI launcher
@@ -48,7 +50,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg2",
-                    choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg4u", "cfg5"])
+                    choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg4u", "cfg5", "latency"])
     ap.add_argument("--mode", default=None, choices=["steps", "fused", "faithful"],
                     help="execution mode of the collective (default: per-step replay)")
     ap.add_argument("--scale", type=float, default=1.0,
@@ -207,10 +209,12 @@ def make_all_gather(P, shard_bytes, mode, device, uneven=False, seed=3):
         return True
 
     payload = sum(nbytes)
-    alg = 2 * payload * P                       # 2 * bytes per materialised output, P outputs
     if kernel == "k_gather_multicast":
+        # every shard is read once and written into each of the P outputs
+        alg = (1 + P) * payload
         kb, kl = alg, 1
     else:
+        alg = 2 * payload * P                   # 2 * bytes per materialised output, P outputs
         kb, kl = 2 * P * shard_bytes, P         # one batched step moves one shard per rank
     info = dict(alg_bytes=alg, kernel=kernel, kernel_bytes=kb, kernel_launches=kl, launches=launches,
                 desc=f"all_gather placement, P={P} virtual ranks, bf16 shards of ~{shard_bytes / MiB:.0f} MiB"
@@ -261,6 +265,43 @@ def build_workload(name, mode, scale, device):
     raise ValueError(name)
 
 
+def latency_sweep(steps, warmup, device):
+    """Microseconds per call for launch-bound message sizes (bf16)."""
+    import torch
+    from pccl import kernels
+
+    def us(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(steps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e3 / steps
+
+    rows = []
+    P = 8
+    for nbytes in [4096 << i for i in range(9)]:            # 4 KiB .. 1 MiB
+        n = nbytes // 2
+        x, y = _randn_bf16(n, 1.0, 1, device), _randn_bf16(n, 1.0, 2, device)
+        z = torch.empty_like(x)
+        B = max(8, n // P)
+        ins = [_randn_bf16(P * B, 1.0, 10 + r, device) for r in range(P)]
+        outs = [torch.empty(B, dtype=torch.bfloat16, device=device) for _ in range(P)]
+        work = [torch.empty_like(t) for t in ins]
+        rows.append({
+            "bytes": nbytes,
+            "accumulate_us": round(us(lambda: kernels.accumulate(x, y)), 2),
+            "copy_us": round(us(lambda: kernels.copy(z, x)), 2),
+            "ring_rs_p8_steps_us": round(us(lambda: kernels.reduce_scatter_ranks(outs, ins, "ring", "steps", work)), 2),
+            "ring_rs_p8_fused_us": round(us(lambda: kernels.reduce_scatter_ranks(outs, ins, "ring", "fused")), 2),
+        })
+    return rows
+
+
 # ---------------------------------------------------------------------------
 # CPU baseline (oracle/cpu_baseline.c), bounded sample
 # ---------------------------------------------------------------------------
@@ -282,8 +323,12 @@ def cpu_baseline(info):
     ranks = min(P, max(1, host_cores))
     if ranks & (ranks - 1):
         ranks = 1 << (ranks.bit_length() - 1)
-    block = (1 << 21) if dtype == "bf16" else (1 << 20)      # 4 MiB blocks
-    args = ["--alg", "ring", "--dtype", dtype, "--block", str(block), "--warmup", "1", "--iters", "5",
+    if info["kernel"] == "k_add_segs" and ranks == info["P"]:
+        block, iters, sample = info["B"], 12, "the workload itself (same P, dtype and block size)"
+    else:
+        block, iters = (1 << 22) if dtype == "bf16" else (1 << 21), 60      # 8 MiB blocks
+        sample = "a ring reduce_scatter of the same dtype with 8 MiB blocks"
+    args = ["--alg", "ring", "--dtype", dtype, "--block", str(block), "--warmup", "1", "--iters", str(iters),
             "--scale", "0.01" if dtype == "bf16" else "1.0"]
     launcher = None
     for cand in ("/opt/conda/bin/mpiexec.hydra", shutil.which("mpiexec.hydra"), shutil.which("mpiexec")):
@@ -297,16 +342,17 @@ def cpu_baseline(info):
     for cmd, transport in attempts:
         try:
             t0 = time.time()
-            p = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+            p = subprocess.run(cmd, capture_output=True, text=True, timeout=400)
             line = [l for l in p.stdout.splitlines() if l.startswith("{")]
             if p.returncode == 0 and line:
                 r = json.loads(line[-1])
                 return {"value": round(r["GBps"], 3), "unit": "GB/s", "cores": ranks, "kind": "port",
                         "ms_per_call": round(r["ms_per_call"], 3), "host_cores": host_cores,
-                        "sample": f"ring reduce_scatter of the reference (pccl/src/reduce_scatter.cpp:101-155) "
-                                  f"on host buffers, {ranks} ranks = {ranks} processes over {transport}, {dtype}, "
-                                  f"{block} elements per block ({ranks * block} per rank), 1 warm-up + 5 timed "
-                                  f"calls, {time.time() - t0:.1f} s wall"}
+                        "sample": f"{sample}: ring reduce_scatter of the reference "
+                                  f"(pccl/src/reduce_scatter.cpp:101-155) on host buffers, {ranks} ranks = {ranks} "
+                                  f"processes over {transport}, {dtype}, {block} elements per block "
+                                  f"({ranks * block} per rank), 1 warm-up + {iters} timed calls, "
+                                  f"{time.time() - t0:.1f} s wall"}
         except Exception:                                     # noqa: BLE001
             continue
     return {"value": None, "unit": "GB/s", "cores": 0, "kind": "port", "sample": "baseline program failed"}
@@ -332,6 +378,19 @@ def main():
         lib.set_tuning(k, int(v))
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
+
+    if args.workload == "latency":
+        rows = latency_sweep(max(args.steps, 50), max(args.warmup, 10), device)
+        last = rows[-1]
+        print(json.dumps({
+            "metric": METRIC, "value": round(3 * last["bytes"] / last["accumulate_us"] / 1e3, 1), "unit": "GB/s",
+            "n_gpus": 1, "steps": max(args.steps, 50), "warmup": max(args.warmup, 10),
+            "ms_per_step": round(last["accumulate_us"] / 1e3, 5), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "latency: bf16 messages of 4 KiB .. 1 MiB; value = accumulate at 1 MiB; "
+                                   "microseconds per call include the Python/ctypes launch path",
+                       "latency_us": rows}, "roofline": None, "cpu_baseline": None}), flush=True)
+        return 0
 
     step, info = build_workload(args.workload, args.mode, args.scale, device)
     torch.cuda.synchronize()

