@@ -9,7 +9,7 @@ algorithmic bytes of that collective divided by its time (GB/s, 1 GB = 1e9 B).
 Timing follows benchmark_raw_collectives/utils.py:16-33 of the reference:
 warm-up calls, then the mean over the timed calls between two device events.
 
-Workloads (BASELINE.json `configs`; `cfg2` is the one the metric is quoted on):
+Workloads (`cfg2` is the one the headline metric is quoted on):
   cfg1  ring reduce_scatter, P=4, fp32, 16 Mi elements per rank
   cfg2  ring reduce_scatter, P=8, bf16, 256 Mi elements per rank, per-hop
         accumulate with bf16 rounding at every hop              (default)
@@ -54,7 +54,7 @@ def parse_args():
     ap.add_argument("--mode", default=None, choices=["steps", "fused", "faithful"],
                     help="execution mode of the collective (default: per-step replay)")
     ap.add_argument("--scale", type=float, default=1.0,
-                    help="shrink the per-rank message by this factor (1.0 = BASELINE size)")
+                    help="shrink the per-rank message by this factor (1.0 = full size)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",

@@ -26,9 +26,9 @@ def inputs(P, n, dtype, seed, kind):
     xs = []
     for r in range(P):
         rng = np.random.default_rng(seed + r)
-        if kind == "uniform":                      # BASELINE config 1: uniform[-1, 1], seed + rank
+        if kind == "uniform":                      # the P=4 fp32 workload: uniform[-1, 1], seed + rank
             x = (rng.random(n, dtype=np.float32) * 2 - 1)
-        elif kind == "grad":                       # BASELINE config 2: normal(0, 1e-2)
+        elif kind == "grad":                       # the P=8 bf16 workload: normal(0, 1e-2)
             x = rng.standard_normal(n, dtype=np.float32) * np.float32(1e-2)
         else:                                      # normal(0, 1)
             x = rng.standard_normal(n, dtype=np.float32)

@@ -44,7 +44,7 @@ def test_reduce_scatter_driver(target, dtype, mode, alg, P):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_config1_shape_small_ring_p4_uniform(target, dtype):
-    """BASELINE config 1 at reduced length: P=4, uniform[-1,1], seed + rank;
+    """The P=4 fp32 workload at reduced length: uniform[-1,1], seed + rank;
     all three modes agree with the oracle and with the closed-form left fold."""
     import torch
     from pccl import kernels

@@ -1,4 +1,4 @@
-"""Parity at BASELINE.json's full sizes (GPU only).
+"""Parity at the full sizes of the benchmark workloads (GPU only).
 
 The numpy oracle cannot chew 4 GiB per test, but every collective here is
 element-wise across ranks: output position i of block j depends only on
