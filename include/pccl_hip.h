@@ -215,6 +215,40 @@ int pccl_hip_all_gather_uneven_virtual(void* const* outputs,
                                        const size_t* dst_off, int P,
                                        void* stream);
 
+/* ---- 2-D (hierarchical) collectives on virtual ranks ------------------------
+ * World of intra*inter ranks, rank w = j*intra + i (node j, local rank i):
+ * the inner group of w is its node {j*intra + i'}, the outer group the ranks
+ * {j'*intra + i} (pccl/process_groups.py:97-98).  Replaces reduce_scatter_2D
+ * (pccl/reduce_scatter.py:205-235): input viewed [inter, intra, m] is permuted
+ * to [intra, inter, m], reduce-scattered inside the node, then across nodes.
+ * The permutation is never materialised: the first inner step reads the inputs
+ * through it (strided pieces).  One launch per step serves ALL groups of a
+ * level, i.e. (intra-1)+(inter-1) launches for "ring".
+ *   inputs[w]  : intra*inter*m elements;  outputs[w] : m elements
+ *   work[w]    : intra*inter*m elements (needed if intra > 2 or inter > 2)
+ *   mid[w]     : inter*m elements (needed if intra > 1 and inter > 1)
+ *   mode       : PCCL_HIP_MODE_STEPS, or PCCL_HIP_MODE_FUSED = ONE launch that
+ *                folds all intra*inter inputs in the two-level order
+ *                (work and mid may then be NULL).
+ * Both levels use `algorithm`; intra*inter <= PCCL_HIP_MAX_RANKS. */
+int pccl_hip_reduce_scatter_2d_virtual(void* const* outputs,
+                                       const void* const* inputs,
+                                       void* const* work, void* const* mid,
+                                       int intra, int inter, size_t m, int dtype,
+                                       const char* algorithm, int mode,
+                                       void* stream);
+
+/* all_gather_2D (pccl/all_gather.py:136-159): gather across nodes, gather
+ * inside the node, un-permute [intra, inter, n] -> [inter, intra, n]; the inner
+ * stage writes through the un-permutation, so no extra pass is made.
+ *   inputs[w]  : block_bytes bytes;  outputs[w] : intra*inter*block_bytes
+ *   mid[w]     : inter*block_bytes bytes (needed if intra > 1 and inter > 1)
+ * PCCL_HIP_MODE_FUSED places every shard directly (one launch). */
+int pccl_hip_all_gather_2d_virtual(void* const* outputs,
+                                   const void* const* inputs, void* const* mid,
+                                   int intra, int inter, size_t block_bytes,
+                                   const char* algorithm, int mode, void* stream);
+
 /* ---- launch tuning (for measurement) ------------------------------------
  * key: "grid_cap" (max workgroups per launch, 0 = one tile per workgroup),
  *      "unroll"   (128-bit vectors per thread per operand: 1, 2, 4 or 8),

@@ -117,28 +117,41 @@ size_t esize_of(int dtype) {
   return dtype == PCCL_HIP_F32 ? 4 : dtype == PCCL_HIP_BF16 ? 2 : 0;
 }
 
+Pieces contiguous(size_t n) {
+  Pieces pc{};
+  pc.s1 = pc.s2 = 1;
+  pc.len = n;
+  return pc;
+}
+
 struct AddLaunch {
   const AddSegs* segs;
   int count, dtype;
-  size_t n, tiles;
+  Pieces pc;
+  size_t tiles;
   hipStream_t stream;
   template <int U, bool NTL, bool NTS>
   void operator()() const {
-    unsigned grid = grid_for((size_t)count * tiles);
+    unsigned grid = grid_for((size_t)count * pc.s1 * pc.s2 * tiles);
     if (dtype == PCCL_HIP_F32)
-      hipLaunchKernelGGL((k_add_segs<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, n, tiles);
+      hipLaunchKernelGGL((k_add_segs<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, pc, tiles);
     else
-      hipLaunchKernelGGL((k_add_segs<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, n, tiles);
+      hipLaunchKernelGGL((k_add_segs<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, pc, tiles);
   }
 };
 
-int launch_add(const AddSegs& segs, int count, size_t n, int dtype, hipStream_t stream,
-               const char* what) {
-  if (n == 0 || count == 0) return PCCL_HIP_OK;
+int launch_add_pieces(const AddSegs& segs, int count, const Pieces& pc, int dtype, hipStream_t stream,
+                      const char* what) {
+  if (pc.len == 0 || count == 0 || pc.s1 == 0 || pc.s2 == 0) return PCCL_HIP_OK;
   Tune t = current_tune();
-  AddLaunch l{&segs, count, dtype, n, tiles_for(n * esize_of(dtype), t.unroll), stream};
+  AddLaunch l{&segs, count, dtype, pc, tiles_for(pc.len * esize_of(dtype), t.unroll), stream};
   with_tuning(t, l);
   return launch_status(what);
+}
+
+int launch_add(const AddSegs& segs, int count, size_t n, int dtype, hipStream_t stream,
+               const char* what) {
+  return launch_add_pieces(segs, count, contiguous(n), dtype, stream, what);
 }
 
 struct CopyLaunch {
@@ -159,6 +172,28 @@ int launch_copy(const CopySegs& segs, int count, hipStream_t stream, const char*
   if (longest == 0 || count == 0) return PCCL_HIP_OK;
   Tune t = current_tune();
   CopyLaunch l{&segs, count, tiles_for(longest, t.unroll), stream};
+  with_tuning(t, l);
+  return launch_status(what);
+}
+
+struct CopyPiecesLaunch {
+  const CopyPairs* segs;
+  int count;
+  Pieces pc;
+  size_t tiles;
+  hipStream_t stream;
+  template <int U, bool NTL, bool NTS>
+  void operator()() const {
+    unsigned grid = grid_for((size_t)count * pc.s1 * pc.s2 * tiles);
+    hipLaunchKernelGGL((k_copy_pieces<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, pc, tiles);
+  }
+};
+
+int launch_copy_pieces(const CopyPairs& segs, int count, const Pieces& pc, hipStream_t stream,
+                       const char* what) {
+  if (pc.len == 0 || count == 0 || pc.s1 == 0 || pc.s2 == 0) return PCCL_HIP_OK;
+  Tune t = current_tune();
+  CopyPiecesLaunch l{&segs, count, pc, tiles_for(pc.len, t.unroll), stream};
   with_tuning(t, l);
   return launch_status(what);
 }
@@ -212,8 +247,8 @@ struct TransposeLaunch {
 // vector per thread ahead of two by 5-10 % for k = 8 and k = 32.
 struct KwayLaunch {
   const KwayArgs* args;
-  int k, nout, dtype, order, first0, per_hop;
-  size_t stride, n;
+  int k, g, nout, dtype, order, first0, per_hop;
+  size_t n;
   hipStream_t stream;
 
   template <class Acc, int U, bool NTL, bool NTS>
@@ -221,7 +256,7 @@ struct KwayLaunch {
     size_t tiles = tiles_for(n * sizeof(typename Acc::op::elem), U);
     unsigned grid = grid_for((size_t)nout * tiles);
 #define PCCL_KWAY(KV) \
-  hipLaunchKernelGGL((k_reduce_kway<Acc, KV, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *args, k, nout, stride, n, first0, tiles)
+  hipLaunchKernelGGL((k_reduce_kway<Acc, KV, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *args, k, g, nout, n, first0, tiles)
     if (order == PCCL_HIP_ORDER_RING) { PCCL_KWAY(0); return; }
     switch (k) {
       case 2: PCCL_KWAY(2); break;
@@ -243,10 +278,11 @@ struct KwayLaunch {
   }
 };
 
-int launch_kway(const KwayArgs& args, int k, int nout, size_t stride, size_t n, int dtype, int order,
+// g = size of the inner groups of a two-level ring order (g >= k: one level).
+int launch_kway(const KwayArgs& args, int k, int g, int nout, size_t n, int dtype, int order,
                 int first0, int per_hop, hipStream_t stream, const char* what) {
   if (n == 0 || nout == 0) return PCCL_HIP_OK;
-  KwayLaunch l{&args, k, nout, dtype, order, first0, per_hop, stride, n, stream};
+  KwayLaunch l{&args, k, g, nout, dtype, order, first0, per_hop, n, stream};
   with_tuning(current_tune(), l);
   return launch_status(what);
 }
@@ -390,7 +426,8 @@ int pccl_hip_reduce_kway(void* out, const void* const* shards, int k, size_t n, 
   KwayArgs args;
   for (int q = 0; q < k; ++q) args.shard[q] = shards[q];
   args.out[0] = out;
-  return launch_kway(args, k, 1, 0, n, dtype, order, first, per_hop_round, (hipStream_t)stream, what);
+  args.eoff[0] = 0;
+  return launch_kway(args, k, k, 1, n, dtype, order, first, per_hop_round, (hipStream_t)stream, what);
 }
 
 int pccl_hip_copy_batched(void* const* dst, const void* const* src, const size_t* nbytes, int count,
@@ -489,9 +526,9 @@ int pccl_hip_reduce_scatter_virtual(void* const* outputs, const void* const* inp
 
   if (mode == PCCL_HIP_MODE_FUSED) {
     KwayArgs args;
-    for (int r = 0; r < P; ++r) { args.shard[r] = inputs[r]; args.out[r] = outputs[r]; }
+    for (int r = 0; r < P; ++r) { args.shard[r] = inputs[r]; args.out[r] = outputs[r]; args.eoff[r] = (size_t)r * B; }
     // ring: block j is folded from rank j+1 on; halving: the butterfly rooted at rank j
-    return launch_kway(args, P, P, B, B, dtype, ring ? PCCL_HIP_ORDER_RING : PCCL_HIP_ORDER_HALVING,
+    return launch_kway(args, P, P, P, B, dtype, ring ? PCCL_HIP_ORDER_RING : PCCL_HIP_ORDER_HALVING,
                        ring ? 1 : 0, 1, st, what);
   }
 
@@ -610,6 +647,272 @@ int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs,
       c.nbytes[r] = block_bytes;
     }
     if (int rc = launch_copy(c, P, st, what)) return rc;
+  }
+  return PCCL_HIP_OK;
+}
+
+int pccl_hip_reduce_scatter_2d_virtual(void* const* outputs, const void* const* inputs,
+                                       void* const* work, void* const* mid, int intra, int inter,
+                                       size_t m, int dtype, const char* algorithm, int mode,
+                                       void* stream) {
+  const char* what = "pccl_hip_reduce_scatter_2d_virtual";
+  if (int rc = check_dtype(dtype, what)) return rc;
+  if (!algorithm) return fail(PCCL_HIP_EINVAL, "%s: algorithm is NULL", what);
+  const bool ring = !strcmp(algorithm, "ring");
+  const bool rec = !strcmp(algorithm, "recursive");
+  if (!ring && !rec)
+    return fail(PCCL_HIP_EINVAL, "Unknown algorithm specified for reduce_scatter_mpi: %s", algorithm);
+  if (intra < 1 || inter < 1 || (long)intra * inter > kMaxSeg)
+    return fail(PCCL_HIP_EINVAL, "%s: intra = %d, inter = %d: need intra, inter >= 1 and intra*inter <= %d",
+                what, intra, inter, kMaxSeg);
+  if (rec && (!pow2(intra) || !pow2(inter)))
+    return fail(PCCL_HIP_EINVAL, "%s: recursive halving needs power-of-two group sizes, got %d x %d", what,
+                intra, inter);
+  if (mode != PCCL_HIP_MODE_STEPS && mode != PCCL_HIP_MODE_FUSED)
+    return fail(PCCL_HIP_EINVAL, "%s: mode %d not offered here (steps or fused)", what, mode);
+  const int W = intra * inter;
+  if (int rc = check_table((const void* const*)outputs, W, what, "outputs")) return rc;
+  if (int rc = check_table(inputs, W, what, "inputs")) return rc;
+  if (m == 0) return PCCL_HIP_OK;
+  hipStream_t st = (hipStream_t)stream;
+  const size_t es = esize_of(dtype);
+  auto at = [es](const void* p, size_t elems) { return (const void*)((const uint8_t*)p + elems * es); };
+  auto atw = [es](void* p, size_t elems) { return (void*)((uint8_t*)p + elems * es); };
+
+  if (W == 1) {
+    CopySegs c;
+    c.dst[0] = outputs[0]; c.src[0] = inputs[0]; c.nbytes[0] = m * es;
+    return launch_copy(c, 1, st, what);
+  }
+
+  if (mode == PCCL_HIP_MODE_FUSED) {
+    KwayArgs args;
+    if (ring) {
+      // world order; block w of every input; inner ring inside each node, then the ring across nodes
+      for (int w = 0; w < W; ++w) { args.shard[w] = inputs[w]; args.out[w] = outputs[w]; args.eoff[w] = (size_t)w * m; }
+      return launch_kway(args, W, inter == 1 ? W : intra, W, m, dtype, PCCL_HIP_ORDER_RING, 1, 1, st, what);
+    }
+    // halving inside the node, then across nodes = ONE butterfly over the index
+    // q = i*inter + j (inner bits above outer bits), rooted at the output's own q
+    for (int j = 0; j < inter; ++j)
+      for (int i = 0; i < intra; ++i) {
+        const int w = j * intra + i, q = i * inter + j;
+        args.shard[q] = inputs[w]; args.out[q] = outputs[w]; args.eoff[q] = (size_t)w * m;
+      }
+    return launch_kway(args, W, W, W, m, dtype, PCCL_HIP_ORDER_HALVING, 0, 1, st, what);
+  }
+
+  const bool need_mid = intra > 1 && inter > 1;
+  const bool need_work = intra > 2 || inter > 2;
+  if (need_mid) if (int rc = check_table((const void* const*)mid, W, what, "mid")) return rc;
+  if (need_work) if (int rc = check_table((const void* const*)work, W, what, "work")) return rc;
+  // result of the inner stage: [inter, m] per rank
+  const void* midr[kMaxSeg];
+  void* midw[kMaxSeg];
+  for (int w = 0; w < W; ++w) {
+    if (intra == 1) { midr[w] = inputs[w]; midw[w] = nullptr; }
+    else if (inter == 1) { midr[w] = outputs[w]; midw[w] = outputs[w]; }
+    else { midr[w] = mid[w]; midw[w] = mid[w]; }
+  }
+  const size_t B1 = (size_t)inter * m;   // inner block: one piece of m per node
+
+  // ---- inner stage: groups of `intra` ranks, inputs read through the permutation ----
+  if (intra > 1 && ring) {
+    for (int s = 0; s < intra - 1; ++s) {
+      AddSegs segs;
+      const bool first = s == 0, last = s == intra - 2;
+      for (int j = 0; j < inter; ++j)
+        for (int i = 0; i < intra; ++i) {
+          const int w = j * intra + i;
+          const int b = ((i - s - 2) % intra + intra) % intra;
+          const int src = j * intra + (i - 1 + intra) % intra;
+          segs.a[w] = at(inputs[w], (size_t)b * m);
+          segs.b[w] = first ? at(inputs[src], (size_t)b * m) : at(work[src], (size_t)b * B1);
+          segs.dst[w] = last ? midw[w] : atw(work[w], (size_t)b * B1);
+        }
+      Pieces pc{};
+      pc.s1 = (unsigned)inter; pc.s2 = 1; pc.len = m;
+      pc.a1 = (size_t)intra * m; pc.b1 = first ? (size_t)intra * m : m; pc.d1 = m;
+      if (int rc = launch_add_pieces(segs, W, pc, dtype, st, what)) return rc;
+    }
+  } else if (intra > 1) {
+    int rounds = 0;
+    while ((1 << rounds) < intra) ++rounds;
+    for (int t = 0; t < rounds; ++t) {
+      AddSegs segs;
+      const int g = intra >> t, half = g / 2;
+      const bool first = t == 0, last = t == rounds - 1;
+      for (int j = 0; j < inter; ++j)
+        for (int i = 0; i < intra; ++i) {
+          const int w = j * intra + i;
+          const bool lower = (i % g) < half;
+          const int p = j * intra + (lower ? i + half : i - half);
+          const size_t b0 = (size_t)(i / g) * g + (lower ? 0 : half);   // first block this rank keeps
+          if (first) {
+            segs.a[w] = at(inputs[w], b0 * m);
+            segs.b[w] = at(inputs[p], b0 * m);
+          } else {
+            segs.a[w] = at(work[w], b0 * B1);
+            segs.b[w] = at(work[p], b0 * B1);
+          }
+          segs.dst[w] = last ? midw[w] : atw(work[w], b0 * B1);
+        }
+      Pieces pc{};
+      if (first) {   // piece (node jj, block bb): strided in the input, contiguous rows in the work layout
+        pc.s1 = (unsigned)inter; pc.s2 = (unsigned)half; pc.len = m;
+        pc.a1 = pc.b1 = (size_t)intra * m; pc.a2 = pc.b2 = m;
+        pc.d1 = m; pc.d2 = B1;
+      } else {
+        pc = contiguous((size_t)half * B1);
+      }
+      if (int rc = launch_add_pieces(segs, W, pc, dtype, st, what)) return rc;
+    }
+  }
+
+  // ---- outer stage: groups of `inter` ranks on the [inter, m] intermediates ----
+  if (inter > 1 && ring) {
+    for (int s = 0; s < inter - 1; ++s) {
+      AddSegs segs;
+      const bool first = s == 0, last = s == inter - 2;
+      for (int j = 0; j < inter; ++j)
+        for (int i = 0; i < intra; ++i) {
+          const int w = j * intra + i;
+          const int b = ((j - s - 2) % inter + inter) % inter;
+          const int src = ((j - 1 + inter) % inter) * intra + i;
+          segs.a[w] = at(midr[w], (size_t)b * m);
+          segs.b[w] = first ? at(midr[src], (size_t)b * m) : at(work[src], (size_t)b * m);
+          segs.dst[w] = last ? outputs[w] : atw(work[w], (size_t)b * m);
+        }
+      if (int rc = launch_add(segs, W, m, dtype, st, what)) return rc;
+    }
+  } else if (inter > 1) {
+    int rounds = 0;
+    while ((1 << rounds) < inter) ++rounds;
+    for (int t = 0; t < rounds; ++t) {
+      AddSegs segs;
+      const int g = inter >> t, half = g / 2;
+      const bool first = t == 0, last = t == rounds - 1;
+      for (int j = 0; j < inter; ++j)
+        for (int i = 0; i < intra; ++i) {
+          const int w = j * intra + i;
+          const bool lower = (j % g) < half;
+          const int p = (lower ? j + half : j - half) * intra + i;
+          const size_t b0 = (size_t)(j / g) * g + (lower ? 0 : half);
+          segs.a[w] = first ? at(midr[w], b0 * m) : at(work[w], b0 * m);
+          segs.b[w] = first ? at(midr[p], b0 * m) : at(work[p], b0 * m);
+          segs.dst[w] = last ? outputs[w] : atw(work[w], b0 * m);
+        }
+      if (int rc = launch_add(segs, W, (size_t)half * m, dtype, st, what)) return rc;
+    }
+  }
+  return PCCL_HIP_OK;
+}
+
+int pccl_hip_all_gather_2d_virtual(void* const* outputs, const void* const* inputs, void* const* mid,
+                                   int intra, int inter, size_t block_bytes, const char* algorithm,
+                                   int mode, void* stream) {
+  const char* what = "pccl_hip_all_gather_2d_virtual";
+  if (!algorithm) return fail(PCCL_HIP_EINVAL, "%s: algorithm is NULL", what);
+  const bool ring = !strcmp(algorithm, "ring");
+  const bool rec = !strcmp(algorithm, "recursive");
+  if (!ring && !rec)
+    return fail(PCCL_HIP_EINVAL, "Unknown algorithm specified for all_gather_mpi: %s", algorithm);
+  if (intra < 1 || inter < 1 || (long)intra * inter > kMaxSeg)
+    return fail(PCCL_HIP_EINVAL, "%s: intra = %d, inter = %d: need intra, inter >= 1 and intra*inter <= %d",
+                what, intra, inter, kMaxSeg);
+  if (rec && (!pow2(intra) || !pow2(inter)))
+    return fail(PCCL_HIP_EINVAL, "%s: recursive doubling needs power-of-two group sizes, got %d x %d", what,
+                intra, inter);
+  if (mode != PCCL_HIP_MODE_STEPS && mode != PCCL_HIP_MODE_FUSED)
+    return fail(PCCL_HIP_EINVAL, "%s: mode %d not offered here (steps or fused)", what, mode);
+  const int W = intra * inter;
+  if (int rc = check_table((const void* const*)outputs, W, what, "outputs")) return rc;
+  if (int rc = check_table(inputs, W, what, "inputs")) return rc;
+  const size_t n = block_bytes;
+  if (n == 0) return PCCL_HIP_OK;
+  hipStream_t st = (hipStream_t)stream;
+
+  if (W == 1) {
+    CopySegs one;
+    one.dst[0] = outputs[0]; one.src[0] = inputs[0]; one.nbytes[0] = n;
+    return launch_copy(one, 1, st, what);
+  }
+
+  if (mode == PCCL_HIP_MODE_FUSED) {   // the 2-D result is the concatenation in world order
+    size_t nbytes[kMaxSeg], off[kMaxSeg];
+    for (int w = 0; w < W; ++w) { nbytes[w] = n; off[w] = (size_t)w * n; }
+    return pccl_hip_all_gather_uneven_virtual(outputs, inputs, nbytes, off, W, stream);
+  }
+
+  const bool need_mid = intra > 1 && inter > 1;
+  if (need_mid) if (int rc = check_table((const void* const*)mid, W, what, "mid")) return rc;
+  // outer result per rank, [inter, n]; with one rank per node it IS the output
+  uint8_t* M[kMaxSeg];
+  for (int w = 0; w < W; ++w)
+    M[w] = inter == 1 ? (uint8_t*)inputs[w] : intra == 1 ? (uint8_t*)outputs[w] : (uint8_t*)mid[w];
+  CopyPairs c;
+
+  // ---- outer stage: gather across nodes into M ----
+  if (inter > 1) {
+    for (int j = 0; j < inter; ++j)
+      for (int i = 0; i < intra; ++i) { const int w = j * intra + i; c.dst[w] = M[w] + (size_t)j * n; c.src[w] = inputs[w]; }
+    if (int rc = launch_copy_pieces(c, W, contiguous(n), st, what)) return rc;
+    if (rec) {
+      for (int seg = 1; seg < inter; seg *= 2) {
+        for (int j = 0; j < inter; ++j)
+          for (int i = 0; i < intra; ++i) {
+            const int w = j * intra + i, pj = j ^ seg, p = pj * intra + i;
+            const int gs = (j / (2 * seg)) * (2 * seg);
+            const size_t off = (size_t)(j < pj ? gs + seg : gs) * n;
+            c.dst[w] = M[w] + off; c.src[w] = M[p] + off;
+          }
+        if (int rc = launch_copy_pieces(c, W, contiguous((size_t)seg * n), st, what)) return rc;
+      }
+    } else {
+      for (int s = 0; s < inter - 1; ++s) {
+        for (int j = 0; j < inter; ++j)
+          for (int i = 0; i < intra; ++i) {
+            const int w = j * intra + i, src = ((j - 1 + inter) % inter) * intra + i;
+            const size_t off = (size_t)(((j - s - 1) % inter + inter) % inter) * n;
+            c.dst[w] = M[w] + off; c.src[w] = M[src] + off;
+          }
+        if (int rc = launch_copy_pieces(c, W, contiguous(n), st, what)) return rc;
+      }
+    }
+  }
+  if (intra == 1) return PCCL_HIP_OK;
+
+  // ---- inner stage: gather inside the node, written through the un-permutation:
+  // inner block ii of the [intra, inter, n] layout is the pieces (jj*intra + ii)*n of the output ----
+  Pieces pc{};
+  pc.s1 = (unsigned)inter; pc.s2 = 1; pc.len = n; pc.d1 = (size_t)intra * n; pc.a1 = n;
+  for (int j = 0; j < inter; ++j)
+    for (int i = 0; i < intra; ++i) { const int w = j * intra + i; c.dst[w] = (uint8_t*)outputs[w] + (size_t)i * n; c.src[w] = M[w]; }
+  if (int rc = launch_copy_pieces(c, W, pc, st, what)) return rc;
+  pc.a1 = (size_t)intra * n;   // from here on both sides are output layouts
+  if (rec) {
+    for (int seg = 1; seg < intra; seg *= 2) {
+      for (int j = 0; j < inter; ++j)
+        for (int i = 0; i < intra; ++i) {
+          const int w = j * intra + i, pi = i ^ seg, p = j * intra + pi;
+          const int gs = (i / (2 * seg)) * (2 * seg);
+          const size_t off = (size_t)(i < pi ? gs + seg : gs) * n;
+          c.dst[w] = (uint8_t*)outputs[w] + off; c.src[w] = (const uint8_t*)outputs[p] + off;
+        }
+      pc.len = (size_t)seg * n;
+      if (int rc = launch_copy_pieces(c, W, pc, st, what)) return rc;
+    }
+  } else {
+    for (int s = 0; s < intra - 1; ++s) {
+      for (int j = 0; j < inter; ++j)
+        for (int i = 0; i < intra; ++i) {
+          const int w = j * intra + i, src = j * intra + (i - 1 + intra) % intra;
+          const size_t off = (size_t)(((i - s - 1) % intra + intra) % intra) * n;
+          c.dst[w] = (uint8_t*)outputs[w] + off; c.src[w] = (const uint8_t*)outputs[src] + off;
+        }
+      pc.len = n;
+      if (int rc = launch_copy_pieces(c, W, pc, st, what)) return rc;
+    }
   }
   return PCCL_HIP_OK;
 }

@@ -301,15 +301,35 @@ struct AddSegs {
   const void* b[kMaxSeg];
 };
 
-// `count` segments of n elements: dst[s] = a[s] + b[s].
+// A segment may consist of s1*s2 pieces of `len` elements (bytes for copies):
+// piece (p1, p2) of operand X starts at X + p1*X1 + p2*X2.  This is how the
+// [inter, intra, m] <-> [intra, inter, m] block permutation of the 2-D
+// collectives is read or written in place instead of being materialised.
+// s1 = s2 = 1 describes a plain contiguous segment.
+struct Pieces {
+  unsigned s1, s2;
+  size_t len;
+  size_t d1, d2;   // destination strides
+  size_t a1, a2;   // first operand (or copy source) strides
+  size_t b1, b2;   // second operand strides
+};
+
+// `count` segments: dst[s] = a[s] + b[s], piece by piece.
 template <class Op, int U, bool NTL, bool NTS>
-__global__ __launch_bounds__(kThreads) void k_add_segs(AddSegs t, int count, size_t n,
-                                                       size_t tiles_per_seg) {
-  const size_t total = (size_t)count * tiles_per_seg;
+__global__ __launch_bounds__(kThreads) void k_add_segs(AddSegs t, int count, Pieces pc,
+                                                       size_t tiles_per_piece) {
+  typedef typename Op::elem elem;
+  const size_t per_seg = (size_t)pc.s1 * pc.s2 * tiles_per_piece;
+  const size_t total = (size_t)count * per_seg;
   for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
-    const int s = (int)(w / tiles_per_seg);
-    const size_t tile = w - (size_t)s * tiles_per_seg;
-    add_tile<Op, U, NTL, NTS>(t.dst[s], t.a[s], t.b[s], n, tile);
+    const int s = (int)(w / per_seg);
+    const size_t rem = w - (size_t)s * per_seg;
+    const size_t piece = rem / tiles_per_piece;
+    const size_t tile = rem - piece * tiles_per_piece;
+    const size_t p1 = piece / pc.s2, p2 = piece - p1 * pc.s2;
+    add_tile<Op, U, NTL, NTS>((elem*)t.dst[s] + p1 * pc.d1 + p2 * pc.d2,
+                              (const elem*)t.a[s] + p1 * pc.a1 + p2 * pc.a2,
+                              (const elem*)t.b[s] + p1 * pc.b1 + p2 * pc.b2, pc.len, tile);
   }
 }
 
@@ -365,6 +385,28 @@ __global__ __launch_bounds__(kThreads) void k_copy_segs(CopySegs t, int count,
     // bytes cover the head shift of the vector body)
     if (tile != 0 && tile * tile_bytes >= nb + 16) continue;
     copy_tile<U, NTL, NTS>(t.dst[s], t.src[s], nb, tile);
+  }
+}
+
+struct CopyPairs {
+  void* dst[kMaxSeg];
+  const void* src[kMaxSeg];
+};
+
+// `count` segments of s1*s2 pieces of pc.len BYTES each (strides in bytes).
+template <int U, bool NTL, bool NTS>
+__global__ __launch_bounds__(kThreads) void k_copy_pieces(CopyPairs t, int count, Pieces pc,
+                                                          size_t tiles_per_piece) {
+  const size_t per_seg = (size_t)pc.s1 * pc.s2 * tiles_per_piece;
+  const size_t total = (size_t)count * per_seg;
+  for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
+    const int s = (int)(w / per_seg);
+    const size_t rem = w - (size_t)s * per_seg;
+    const size_t piece = rem / tiles_per_piece;
+    const size_t tile = rem - piece * tiles_per_piece;
+    const size_t p1 = piece / pc.s2, p2 = piece - p1 * pc.s2;
+    copy_tile<U, NTL, NTS>((uint8_t*)t.dst[s] + p1 * pc.d1 + p2 * pc.d2,
+                           (const uint8_t*)t.src[s] + p1 * pc.a1 + p2 * pc.a2, pc.len, tile);
   }
 }
 
@@ -434,6 +476,7 @@ __global__ __launch_bounds__(kThreads) void k_block_transpose(uint8_t* dst, cons
 struct KwayArgs {
   const void* shard[kMaxSeg];
   void* out[kMaxSeg];
+  size_t eoff[kMaxSeg];   // element offset into every shard, per output
 };
 
 // S(M, H) of the halving butterfly over K leaves v[m] = shard[first ^ m]:
@@ -454,34 +497,61 @@ __device__ __forceinline__ void tree_sum(Load& load, int first, float* out) {
   }
 }
 
+// Left fold over `count` operands in cyclic order first, first+1, ...; loads
+// are issued in batches of eight ahead of the adds.  load(q, f) fills the L
+// fp32 lanes of operand q; acc receives the result.
+template <class Acc, int L, class Load>
+__device__ __forceinline__ void ring_fold(Load&& load, int count, int first, float* acc) {
+  int q = first;
+  load(q, acc);
+  int done = 1;
+  for (; done + 8 <= count; done += 8) {
+    float f[8][L];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      q = q + 1 == count ? 0 : q + 1;
+      load(q, f[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) Acc::template hop_lanes<L>(acc, f[i]);
+  }
+  for (; done < count; ++done) {
+    q = q + 1 == count ? 0 : q + 1;
+    float f[L];
+    load(q, f);
+    Acc::template hop_lanes<L>(acc, f);
+  }
+}
+
 // Fold the k shards at one position in the order of a schedule.
-//   K == 0 : ring order, runtime k: first, first+1, ... (mod k), loads issued
-//            in batches of eight ahead of the adds
+//   K == 0 : ring order, runtime k (one level if g >= k, else two levels)
 //   K >= 2 : halving order for k == K: leaves v[m] = shard[first ^ m] summed by
 //            the butterfly v[m] += v[m+h], h = K/2 .. 1, evaluated depth first
 //            by tree_sum (the same tree with only log2 K live partial sums).
-// load(q, f) fills the L fp32 lanes of shard q; acc receives the result.
 template <class Acc, int K, int L, class Load>
-__device__ __forceinline__ void fold_shards(Load&& load, int k, int first, float* acc) {
+__device__ __forceinline__ void fold_shards(Load&& load, int k, int g, int first, int first_outer,
+                                            float* acc) {
   if constexpr (K == 0) {
-    int q = first;
-    load(q, acc);
-    int done = 1;
-    for (; done + 8 <= k; done += 8) {
-      float f[8][L];
+    if (g >= k) {
+      ring_fold<Acc, L>(load, k, first, acc);
+    } else {
+      // two-level ring: shards form k/g groups of g; every group is folded in
+      // ring order from `first`, and the group sums are folded in ring order
+      // from group `first_outer` (inner, then outer reduce_scatter of the 2-D
+      // collective)
+      const int groups = k / g;
+      int go = first_outer;
+      for (int og = 0; og < groups; ++og) {
+        float part[L];
+        ring_fold<Acc, L>([&](int q, float* f) { load(go * g + q, f); }, g, first, part);
+        if (og == 0) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        q = q + 1 == k ? 0 : q + 1;
-        load(q, f[i]);
+          for (int l = 0; l < L; ++l) acc[l] = part[l];
+        } else {
+          Acc::template hop_lanes<L>(acc, part);
+        }
+        go = go + 1 == groups ? 0 : go + 1;
       }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) Acc::template hop_lanes<L>(acc, f[i]);
-    }
-    for (; done < k; ++done) {
-      q = q + 1 == k ? 0 : q + 1;
-      float f[L];
-      load(q, f);
-      Acc::template hop_lanes<L>(acc, f);
     }
   } else {
     tree_sum<Acc, K, 0, 1, L>(load, first, acc);
@@ -489,13 +559,14 @@ __device__ __forceinline__ void fold_shards(Load&& load, int k, int first, float
 }
 
 // Fused k-way reduce, one pass: output j = fold over the k shards of
-// shard[.][j*stride + i], i < n, starting the schedule at shard
-// (first0 + j) mod k.  The vector path needs 16-byte aligned operands;
+// shard[.][eoff[j] + i], i < n, starting the schedule at shard
+// (first0 + j) mod k (or, for the two-level ring, at the inner and outer
+// successors of j).  The vector path needs 16-byte aligned operands;
 // otherwise (and for the last n % kPerVec elements) elements go one by one
 // through the same fold.
 template <class Acc, int K, int U, bool NTL, bool NTS>
-__global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int nout,
-                                                          size_t stride, size_t n, int first0,
+__global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int g, int nout,
+                                                          size_t n, int first0,
                                                           size_t tiles_per_seg) {
   typedef typename Acc::op Op;
   typedef typename Op::elem elem;
@@ -505,8 +576,11 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
   for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
     const int j = (int)(w / tiles_per_seg);
     const size_t tile = w - (size_t)j * tiles_per_seg;
-    const int first = (first0 + j) % k;
-    const size_t eoff = (size_t)j * stride;
+    // flat: the schedule of output j starts at shard (first0 + j) mod k;
+    // two-level ring (g < k): inner start (j mod g) + 1, outer start (j / g) + 1
+    const int first = g >= k ? (first0 + j) % k : (j % g + 1) % g;
+    const int first_outer = g >= k ? 0 : (j / g + 1) % (k / g);
+    const size_t eoff = t.eoff[j];
     elem* out = (elem*)t.out[j];
 
     bool aligned = (((uintptr_t)out) & 15u) == 0;
@@ -524,7 +598,7 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
             [&](int q, float* f) {
               Acc::widen(ld16<NTL>((const u32x4*)((const elem*)t.shard[q] + eoff) + v), f);
             },
-            k, first, acc);
+            k, g, first, first_outer, acc);
         st16<NTS>((u32x4*)out + v, Acc::narrow(acc));
       }
     }
@@ -547,7 +621,7 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
             if constexpr (sizeof(elem) == 4) f[0] = e;
             else f[0] = __uint_as_float((uint32_t)e << 16);
           },
-          k, first, acc1);
+          k, g, first, first_outer, acc1);
       if constexpr (sizeof(elem) == 4) out[i] = acc1[0];
       else out[i] = (elem)(bf16_round_hi(acc1[0]) >> 16);
     }

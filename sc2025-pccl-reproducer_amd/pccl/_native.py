@@ -53,6 +53,9 @@ SIGNATURES = {
     "pccl_hip_reduce_scatter_virtual": (_int, [_vpp, _vpp, _vpp, _int, _sz, _int, ctypes.c_char_p, _int, _vp]),
     "pccl_hip_all_gather_virtual": (_int, [_vpp, _vpp, _int, _sz, ctypes.c_char_p, _int, _vp]),
     "pccl_hip_all_gather_uneven_virtual": (_int, [_vpp, _vpp, _szp, _szp, _int, _vp]),
+    "pccl_hip_reduce_scatter_2d_virtual": (_int, [_vpp, _vpp, _vpp, _vpp, _int, _int, _sz, _int, ctypes.c_char_p,
+                                                  _int, _vp]),
+    "pccl_hip_all_gather_2d_virtual": (_int, [_vpp, _vpp, _vpp, _int, _int, _sz, ctypes.c_char_p, _int, _vp]),
     "pccl_hip_set_tuning": (_int, [ctypes.c_char_p, ctypes.c_long]),
     "pccl_hip_get_tuning": (ctypes.c_long, [ctypes.c_char_p]),
 }
@@ -161,6 +164,19 @@ class NativeLib:
         P = len(inputs)
         self._check(self._lib.pccl_hip_all_gather_uneven_virtual(
             _ptr_table(outputs), _ptr_table(inputs), _size_table(nbytes), _size_table(dst_off), P, stream))
+
+
+    def reduce_scatter_2d_virtual(self, outputs, inputs, work, mid, intra, inter, m, dtype, algorithm,
+                                  mode=MODE_STEPS, stream=0):
+        self._check(self._lib.pccl_hip_reduce_scatter_2d_virtual(
+            _ptr_table(outputs), _ptr_table(inputs), _ptr_table(work), _ptr_table(mid), intra, inter, m, dtype,
+            algorithm.encode(), mode, stream))
+
+    def all_gather_2d_virtual(self, outputs, inputs, mid, intra, inter, block_bytes, algorithm,
+                              mode=MODE_STEPS, stream=0):
+        self._check(self._lib.pccl_hip_all_gather_2d_virtual(
+            _ptr_table(outputs), _ptr_table(inputs), _ptr_table(mid), intra, inter, block_bytes,
+            algorithm.encode(), mode, stream))
 
 
 _lock = threading.Lock()

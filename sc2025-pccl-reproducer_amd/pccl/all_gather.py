@@ -95,6 +95,11 @@ def all_gather_2D(output_tensor: torch.Tensor,
     assert input_tensor.dim() == 1 and output_tensor.dim() == 1, "all_gather_2D only admits 1D tensors"
     intra_node_group_size, inter_node_group_size = group.get_world_size()
 
+    if use_pccl_cpp_backend and getattr(group, "virtual_world", None) is not None:
+        # virtual ranks, native backend: both levels and the un-permutation in one batched call
+        ext.all_gather_2d(output_tensor, input_tensor, group, "recursive" if use_rd else "ring")
+        return
+
     output_intermediate = torch.empty(input_tensor.size(0) * inter_node_group_size,
                                       device=input_tensor.device, dtype=input_tensor.dtype)
     _all_gather(output_intermediate, input_tensor, group.get_outer_group(), async_op=False,

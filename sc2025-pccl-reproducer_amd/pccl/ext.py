@@ -87,3 +87,50 @@ def all_gather_mpi(output_tensor: torch.Tensor, input_tensor: torch.Tensor, py_c
         kernels.all_gather_ranks([p[0] for p in payloads], [p[1] for p in payloads], algorithm)
 
     py_comm._collective(f"all_gather_mpi[{algorithm}]", (output_tensor, input_tensor), launch)
+
+
+def _run_grids(payloads, intra, inter, launch_grid):
+    """Split the world into its independent intra*inter grids (consecutive
+    ranks, pccl/process_groups.py:97-98) and launch each."""
+    per = intra * inter
+    for g0 in range(0, len(payloads), per):
+        part = payloads[g0:g0 + per]
+        launch_grid([p[0] for p in part], [p[1] for p in part])
+
+
+def reduce_scatter_2d(output_tensor: torch.Tensor, input_tensor: torch.Tensor, groups, algorithm: str) -> None:
+    """Native path of reduce_scatter_2D on virtual ranks: every rank of the world
+    communicator brings its tensors; the last one enqueues the batched launches
+    (include/pccl_hip.h: pccl_hip_reduce_scatter_2d_virtual)."""
+    intra, inter = groups.grid_shape
+    world = groups.virtual_world
+    if input_tensor.numel() % (intra * inter):
+        raise RuntimeError("Input tensor size must be divisible by number of processes")
+    if output_tensor.numel() != input_tensor.numel() // (intra * inter):
+        raise RuntimeError("Output tensor must have block_size elements (input tensor numel()/world_size)")
+    kernels.check_device_tensor(input_tensor, "input")
+    kernels.check_device_tensor(output_tensor, "output")
+
+    def launch(payloads):
+        _run_grids(payloads, intra, inter,
+                   lambda outs, ins: kernels.reduce_scatter_2d_ranks(outs, ins, intra, inter, algorithm))
+
+    world._collective(f"reduce_scatter_2D[{algorithm}]", (output_tensor, input_tensor), launch)
+
+
+def all_gather_2d(output_tensor: torch.Tensor, input_tensor: torch.Tensor, groups, algorithm: str) -> None:
+    """Native path of all_gather_2D on virtual ranks (pccl_hip_all_gather_2d_virtual)."""
+    intra, inter = groups.grid_shape
+    world = groups.virtual_world
+    if input_tensor.dtype != output_tensor.dtype:
+        raise RuntimeError("Input and output tensors must have the same dtype.")
+    if output_tensor.numel() != input_tensor.numel() * intra * inter:
+        raise RuntimeError("Output tensor must have total_elem elements (input tensor numel() *world_size)")
+    kernels.check_device_tensor(input_tensor, "input")
+    kernels.check_device_tensor(output_tensor, "output")
+
+    def launch(payloads):
+        _run_grids(payloads, intra, inter,
+                   lambda outs, ins: kernels.all_gather_2d_ranks(outs, ins, intra, inter, algorithm))
+
+    world._collective(f"all_gather_2D[{algorithm}]", (output_tensor, input_tensor), launch)

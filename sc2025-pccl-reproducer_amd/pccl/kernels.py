@@ -277,3 +277,73 @@ def all_gather_uneven_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[to
     _native.load().all_gather_uneven_virtual(_ptrs(outputs), _ptrs(inputs), nbytes, list(dst_off),
                                              stream_handle())
     return list(dst_off)
+
+
+# ---------------------------------------------------------------------------
+# 2-D (hierarchical) collectives over intra*inter virtual ranks, world order
+# ---------------------------------------------------------------------------
+
+def _check_2d(outputs, inputs, intra, inter):
+    W = intra * inter
+    if intra < 1 or inter < 1 or len(inputs) != W or len(outputs) != W:
+        raise ValueError("need intra*inter inputs and outputs, in world-rank order")
+    if W > MAX_RANKS:
+        raise RuntimeError(f"at most {MAX_RANKS} virtual ranks per 2-D grid")
+    for t in inputs:
+        check_device_tensor(t, "input")
+    for t in outputs:
+        check_device_tensor(t, "output")
+    _same_device(list(inputs) + list(outputs))
+    return W
+
+
+def reduce_scatter_2d_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[torch.Tensor], intra: int,
+                            inter: int, algorithm: str = "recursive", mode=None) -> None:
+    """reduce_scatter_2D for a whole grid of intra*inter virtual ranks (rank
+    w = node*intra + local) in one call: the input permutation of
+    pccl/reduce_scatter.py:226 is read in place by the first inner step, and one
+    launch per step serves every inner (then every outer) group."""
+    W = _check_2d(outputs, inputs, intra, inter)
+    total, dt = inputs[0].numel(), inputs[0].dtype
+    if total % W:
+        raise RuntimeError("Input tensor size must be divisible by number of processes")
+    m = total // W
+    for i, o in zip(inputs, outputs):
+        if i.numel() != total or i.dtype != dt:
+            raise RuntimeError("all ranks must pass inputs of the same dtype and size")
+        if o.numel() != m or o.dtype != dt:
+            raise RuntimeError("Output tensor must have block_size elements (input tensor numel()/world_size)")
+    code = mode_code(mode)
+    if code == MODE_FAITHFUL:
+        code = MODE_STEPS
+    work = mid = None
+    if code == MODE_STEPS:
+        if intra > 2 or inter > 2:
+            work = [torch.empty_like(inputs[w]) for w in range(W)]
+        if intra > 1 and inter > 1:
+            mid = [torch.empty(inter * m, dtype=dt, device=inputs[0].device) for _ in range(W)]
+    _native.load().reduce_scatter_2d_virtual(_ptrs(outputs), _ptrs(inputs), _ptrs(work), _ptrs(mid), intra, inter,
+                                             m, dtype_code(dt), algorithm, code, stream_handle())
+
+
+def all_gather_2d_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[torch.Tensor], intra: int,
+                        inter: int, algorithm: str = "recursive", mode=None) -> None:
+    """all_gather_2D for a whole grid of intra*inter virtual ranks in one call;
+    the inner stage writes through the un-permutation of pccl/all_gather.py:158-159."""
+    W = _check_2d(outputs, inputs, intra, inter)
+    n, dt = inputs[0].numel(), inputs[0].dtype
+    for i, o in zip(inputs, outputs):
+        if i.numel() != n or i.dtype != dt:
+            raise RuntimeError("all ranks must pass shards of the same dtype and size")
+        if o.dtype != dt:
+            raise RuntimeError("Input and output tensors must have the same dtype.")
+        if o.numel() != n * W:
+            raise RuntimeError("Output tensor must have total_elem elements (input tensor numel() *world_size)")
+    code = mode_code(mode)
+    if code == MODE_FAITHFUL:
+        code = MODE_STEPS
+    mid = None
+    if code == MODE_STEPS and intra > 1 and inter > 1:
+        mid = [torch.empty(inter * n, dtype=dt, device=inputs[0].device) for _ in range(W)]
+    _native.load().all_gather_2d_virtual(_ptrs(outputs), _ptrs(inputs), _ptrs(mid), intra, inter,
+                                         n * inputs[0].element_size(), algorithm, code, stream_handle())

@@ -47,6 +47,10 @@ class ProcessGroups:
     ):
         if comm is None:
             assert dist.is_initialized(), "pytorch distributed should be initialized by the user"
+        # virtual ranks: the communicator spanning every grid, and the grid shape,
+        # let the 2-D collectives batch all groups of a level into one launch
+        self.virtual_world = comm
+        self.grid_shape = (intra_group_size, inter_group_size)
         self.inner_group, self.outer_group = self.create_2D_grid(
             intra_group_size=intra_group_size,
             inter_group_size=inter_group_size,

@@ -163,6 +163,12 @@ def reduce_scatter_2D(output_tensor: torch.Tensor,
     assert input_tensor.dim() == 1 and output_tensor.dim() == 1, "all_gather_2D only admits 1D tensors"
     intra_node_group_size, inter_node_group_size = group.get_world_size()
 
+    if use_pccl_cpp_backend and getattr(group, "virtual_world", None) is not None:
+        # virtual ranks, native backend: both levels and the permutation in one
+        # batched call, nothing materialised in between
+        ext.reduce_scatter_2d(output_tensor, input_tensor, group, "recursive" if use_rh else "ring")
+        return
+
     input_permuted = torch.empty_like(input_tensor)
     kernels.block_transpose(input_permuted, input_tensor, inter_node_group_size, intra_node_group_size)
 

@@ -276,6 +276,86 @@ def test_all_gather_2D(target, intra, inter, use_rd, cpp):
         assert torch.equal(t_out[r], cat)      # the 2-D all_gather is a plain concatenation
 
 
+GRIDS = [(1, 1), (2, 1), (1, 2), (2, 2), (4, 2), (2, 4), (3, 2), (2, 3), (1, 8), (8, 1), (4, 4), (8, 8), (16, 4)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("intra,inter", GRIDS)
+@pytest.mark.parametrize("alg", ["ring", "recursive"])
+@pytest.mark.parametrize("mode", ["steps", "fused"])
+def test_reduce_scatter_2d_driver(target, dtype, intra, inter, alg, mode):
+    """The whole 2-D collective in one call: permutation read in place, all
+    groups of a level in one launch, or everything in one fused launch."""
+    import torch
+    from pccl import kernels
+    if alg == "recursive" and ((intra & (intra - 1)) or (inter & (inter - 1))):
+        pytest.skip("halving needs power-of-two groups")
+    W = intra * inter
+    m = 261 if W <= 16 else 37
+    print(f"reduce_scatter_2d {intra}x{inter} alg={alg} mode={mode} dtype={dtype}", flush=True)
+    ins = make_inputs(W, W * m, dtype, seed=61)
+    t_in = [to_torch(x, dtype, target.device) for x in ins]
+    t_out = [torch.zeros(m, dtype=_tdtype(dtype), device=target.device) for _ in range(W)]
+    kernels.reduce_scatter_2d_ranks(t_out, t_in, intra, inter, alg, mode)
+    target.sync()
+    want = O.reduce_scatter_2d(ins, intra, inter, dtype, alg)
+    for w in range(W):
+        assert_bits_equal(to_numpy(t_out[w], dtype), want[w], f"rank {w}")
+        assert_bits_equal(to_numpy(t_in[w], dtype), ins[w], f"input of rank {w} modified")
+
+
+@pytest.mark.parametrize("intra,inter", GRIDS)
+@pytest.mark.parametrize("alg", ["ring", "recursive"])
+@pytest.mark.parametrize("mode", ["steps", "fused"])
+def test_all_gather_2d_driver(target, intra, inter, alg, mode):
+    import torch
+    from pccl import kernels
+    if alg == "recursive" and ((intra & (intra - 1)) or (inter & (inter - 1))):
+        pytest.skip("doubling needs power-of-two groups")
+    W = intra * inter
+    n = 1030 if W <= 16 else 70
+    rng = np.random.default_rng(71)
+    ins = [rng.integers(0, 256, n, dtype=np.uint8) for _ in range(W)]
+    t_in = [torch.from_numpy(x).to(target.device) for x in ins]
+    t_out = [torch.full((W * n,), 0xA5, dtype=torch.uint8, device=target.device) for _ in range(W)]
+    kernels.all_gather_2d_ranks(t_out, t_in, intra, inter, alg, mode)
+    target.sync()
+    want = O.all_gather_2d(ins, intra, inter, alg)
+    for w in range(W):
+        assert np.array_equal(t_out[w].cpu().numpy(), want[w]), f"rank {w}"
+
+
+@pytest.mark.parametrize("mode", ["steps", "fused"])
+def test_2d_per_rank_api_with_two_grids(target, mode, monkeypatch):
+    """world = 2 grids of 2x2: every grid is an independent 2-D collective."""
+    import torch
+    import pccl
+    monkeypatch.setenv("PCCL_VIRTUAL_MODE", mode)
+    intra, inter, grids = 2, 2, 2
+    world_size = intra * inter * grids
+    m = 129
+    ins = make_inputs(world_size, intra * inter * m, O.BF16, seed=81)
+    t_in = [to_torch(x, O.BF16, target.device) for x in ins]
+    t_out = [torch.zeros(m, dtype=torch.bfloat16, device=target.device) for _ in range(world_size)]
+    g_out = [torch.zeros(intra * inter * m, dtype=torch.bfloat16, device=target.device) for _ in range(world_size)]
+    world = pccl.VirtualWorld(world_size, target.device)
+
+    def rank_main(comm):
+        r = comm.Get_rank()
+        pg = pccl.ProcessGroups(intra, inter, inner_group_backend="mpi", outer_group_backend="mpi", comm=comm)
+        pccl.reduce_scatter_2D(t_out[r], t_in[r], group=pg, use_rh=True, use_pccl_cpp_backend=True)
+        pccl.all_gather_2D(g_out[r], t_out[r], group=pg, use_rd=True, use_pccl_cpp_backend=True)
+
+    world.run(rank_main)
+    target.sync()
+    per = intra * inter
+    for g in range(grids):
+        want = O.reduce_scatter_2d(ins[g * per:(g + 1) * per], intra, inter, O.BF16, "recursive")
+        for k in range(per):
+            assert_bits_equal(to_numpy(t_out[g * per + k], O.BF16), want[k], f"grid {g} rank {k}")
+            assert_bits_equal(to_numpy(g_out[g * per + k], O.BF16), np.concatenate(want), f"gather grid {g} rank {k}")
+
+
 @pytest.mark.parametrize("rec", [True, False])
 def test_all_reduce(target, rec):
     import torch
