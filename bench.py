@@ -18,6 +18,8 @@ Workloads (`cfg2` is the one the headline metric is quoted on):
   cfg4  all_gather placement, P=16, bf16 shards of 128 MiB into 2 GiB outputs
   cfg4u the same with uneven shards padded to 256 bytes
   cfg5  fused one-pass reduce of 32 fp32 shards of 32 Mi elements
+  ceilings  what the device sustains for plain streams of 1 GiB: read-only,
+        write-only, copy and 2-reads-1-write add (the practical roofline)
   latency  small messages, 4 KiB .. 1 MiB in bf16: microseconds per accumulate,
         per copy and per whole P=8 ring reduce_scatter (per-step and fused)
 
@@ -50,7 +52,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg2",
-                    choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg4u", "cfg5", "latency"])
+                    choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg4u", "cfg5", "latency", "ceilings"])
     ap.add_argument("--mode", default=None, choices=["steps", "fused", "faithful"],
                     help="execution mode of the collective (default: per-step replay)")
     ap.add_argument("--scale", type=float, default=1.0,
@@ -265,6 +267,40 @@ def build_workload(name, mode, scale, device):
     raise ValueError(name)
 
 
+def ceilings(steps, warmup, device):
+    """GB/s of pure read, pure write, copy and add streams over 1 GiB buffers."""
+    import torch
+    from pccl import _native, kernels
+    lib = _native.load()
+    n = 1 << 30
+    a = torch.zeros(n, dtype=torch.uint8, device=device)
+    b = torch.zeros(n, dtype=torch.uint8, device=device)
+    c = torch.zeros(n, dtype=torch.uint8, device=device)
+    fa, fb, fc = (t.view(torch.float32) for t in (a, b, c))
+
+    def gbps(fn, nbytes):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(steps):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return round(nbytes / (s.elapsed_time(e) / steps * 1e-3) / 1e9, 1)
+
+    st = kernels.stream_handle()
+    return {
+        "read_only": gbps(lambda: lib.probe_stream(0, a.data_ptr(), n, st), n),
+        "write_only": gbps(lambda: lib.probe_stream(1, c.data_ptr(), n, st), n),
+        "copy": gbps(lambda: kernels.copy(c, a), 2 * n),
+        "add_2r1w_f32": gbps(lambda: kernels.add(fc, fa, fb), 3 * n),
+        "torch_copy_": gbps(lambda: c.copy_(a), 2 * n),
+        "torch_add_f32": gbps(lambda: torch.add(fa, fb, out=fc), 3 * n),
+    }
+
+
 def latency_sweep(steps, warmup, device):
     """Microseconds per call for launch-bound message sizes (bf16)."""
     import torch
@@ -378,6 +414,16 @@ def main():
         lib.set_tuning(k, int(v))
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
+
+    if args.workload == "ceilings":
+        res = ceilings(args.steps, args.warmup, device)
+        print(json.dumps({
+            "metric": METRIC, "value": res["add_2r1w_f32"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(3 * (1 << 30) / res["add_2r1w_f32"] / 1e6, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "ceilings: plain streams over 1 GiB buffers; value = the library's add kernel",
+                       "GBps": res}, "roofline": None, "cpu_baseline": None}), flush=True)
+        return 0
 
     if args.workload == "latency":
         rows = latency_sweep(max(args.steps, 50), max(args.warmup, 10), device)

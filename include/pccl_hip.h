@@ -249,6 +249,15 @@ int pccl_hip_all_gather_2d_virtual(void* const* outputs,
                                    int intra, int inter, size_t block_bytes,
                                    const char* algorithm, int mode, void* stream);
 
+/* ---- bandwidth probe (for measurement) --------------------------------------
+ * One pure streaming pass over buf[0:nbytes] with the access shape of the
+ * kernels above: kind 0 reads every byte (nothing is written), kind 1
+ * overwrites every byte with the bf16 pattern of 1.0.  Timing it gives the
+ * read and write bandwidth this device actually sustains, the practical
+ * ceiling the 2-reads-1-write kernels are judged against.  No counterpart in
+ * the reference.  buf must be 16-byte aligned, nbytes >= 4096. */
+int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream);
+
 /* ---- launch tuning (for measurement) ------------------------------------
  * key: "grid_cap" (max workgroups per launch, 0 = one tile per workgroup),
  *      "unroll"   (128-bit vectors per thread per operand: 1, 2, 4 or 8),

@@ -917,4 +917,22 @@ int pccl_hip_all_gather_2d_virtual(void* const* outputs, const void* const* inpu
   return PCCL_HIP_OK;
 }
 
+int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream) {
+  const char* what = "pccl_hip_probe_stream";
+  if (kind != 0 && kind != 1) return fail(PCCL_HIP_EINVAL, "%s: kind must be 0 (read) or 1 (write)", what);
+  if (nbytes < 4096) return fail(PCCL_HIP_EINVAL, "%s: buffer must hold at least 4096 bytes", what);
+  if (!buf || ((uintptr_t)buf & 15u)) return fail(PCCL_HIP_EINVAL, "%s: buffer must be 16-byte aligned", what);
+  const size_t nvec = nbytes / 16;
+  const size_t tiles = (nvec + (size_t)kThreads * 4 - 1) / ((size_t)kThreads * 4);
+  if (tiles > kMaxGrid) return fail(PCCL_HIP_EINVAL, "%s: buffer too large", what);
+  hipStream_t st = (hipStream_t)stream;
+  if (kind == 0)
+    hipLaunchKernelGGL((k_probe_read<4, true>), dim3((unsigned)tiles), dim3(kThreads), 0, st,
+                       (const u32x4*)buf, (u32x4*)buf, nvec);
+  else
+    hipLaunchKernelGGL((k_probe_write<4, false>), dim3((unsigned)tiles), dim3(kThreads), 0, st, (u32x4*)buf,
+                       nvec, 0x3f803f80u);
+  return launch_status(what);
+}
+
 }  // extern "C"

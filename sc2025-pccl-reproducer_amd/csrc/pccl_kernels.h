@@ -473,6 +473,37 @@ __global__ __launch_bounds__(kThreads) void k_block_transpose(uint8_t* dst, cons
   }
 }
 
+// Streaming probes: what this device sustains for a pure read and a pure
+// write stream with the same access shape as the kernels above.  The read
+// probe folds its data with xor and stores only if the result hits a value
+// that zero-filled or random buffers never produce, so the loads stay live.
+template <int U, bool NTL>
+__global__ __launch_bounds__(kThreads) void k_probe_read(const u32x4* src, u32x4* sink, size_t nvec) {
+  const size_t base = (size_t)blockIdx.x * (kThreads * U) + threadIdx.x;
+  u32x4 x[U];
+#pragma unroll
+  for (int j = 0; j < U; ++j) {
+    const size_t v = base + (size_t)j * kThreads;
+    x[j] = v < nvec ? ld16<NTL>(src + v) : u32x4{0, 0, 0, 0};
+  }
+  u32x4 acc = x[0];
+#pragma unroll
+  for (int j = 1; j < U; ++j) acc ^= x[j];
+  if (acc.x == 0x9e3779b9u && acc.y == 0x7f4a7c15u && acc.z == 0xf39cc060u && acc.w == 0x5cedc834u)
+    sink[threadIdx.x] = acc;
+}
+
+template <int U, bool NTS>
+__global__ __launch_bounds__(kThreads) void k_probe_write(u32x4* dst, size_t nvec, uint32_t value) {
+  const size_t base = (size_t)blockIdx.x * (kThreads * U) + threadIdx.x;
+  const u32x4 v4 = {value, value, value, value};
+#pragma unroll
+  for (int j = 0; j < U; ++j) {
+    const size_t v = base + (size_t)j * kThreads;
+    if (v < nvec) st16<NTS>(dst + v, v4);
+  }
+}
+
 struct KwayArgs {
   const void* shard[kMaxSeg];
   void* out[kMaxSeg];

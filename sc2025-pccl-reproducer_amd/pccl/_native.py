@@ -56,6 +56,7 @@ SIGNATURES = {
     "pccl_hip_reduce_scatter_2d_virtual": (_int, [_vpp, _vpp, _vpp, _vpp, _int, _int, _sz, _int, ctypes.c_char_p,
                                                   _int, _vp]),
     "pccl_hip_all_gather_2d_virtual": (_int, [_vpp, _vpp, _vpp, _int, _int, _sz, ctypes.c_char_p, _int, _vp]),
+    "pccl_hip_probe_stream": (_int, [_int, _vp, _sz, _vp]),
     "pccl_hip_set_tuning": (_int, [ctypes.c_char_p, ctypes.c_long]),
     "pccl_hip_get_tuning": (ctypes.c_long, [ctypes.c_char_p]),
 }
@@ -177,6 +178,10 @@ class NativeLib:
         self._check(self._lib.pccl_hip_all_gather_2d_virtual(
             _ptr_table(outputs), _ptr_table(inputs), _ptr_table(mid), intra, inter, block_bytes,
             algorithm.encode(), mode, stream))
+
+
+    def probe_stream(self, kind, buf, nbytes, stream=0):
+        self._check(self._lib.pccl_hip_probe_stream(kind, buf, nbytes, stream))
 
 
 _lock = threading.Lock()

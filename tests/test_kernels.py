@@ -238,3 +238,20 @@ def test_invalid_arguments_return_codes(target):
         target.native.reduce_scatter_virtual([16], [16], None, 4, 0, "tree")
     with pytest.raises(NativeError, match="power-of-two"):
         target.native.reduce_scatter_virtual([16] * 3, [16] * 3, [16] * 3, 4, 0, "recursive")
+
+
+def test_probe_streams(target):
+    """The read probe leaves the buffer alone; the write probe fills it with bf16 1.0."""
+    import torch
+    n = 70_000
+    buf = torch.arange(n, dtype=torch.int32, device=target.device)
+    before = buf.clone()
+    target.native.probe_stream(0, buf.data_ptr(), n * 4, target.stream())
+    target.sync()
+    assert torch.equal(buf, before)
+    target.native.probe_stream(1, buf.data_ptr(), n * 4, target.stream())
+    target.sync()
+    assert bool((buf.view(torch.int16) == 0x3F80).all())
+    from pccl._native import NativeError
+    with pytest.raises(NativeError, match="kind must be"):
+        target.native.probe_stream(2, buf.data_ptr(), n * 4, target.stream())
