@@ -328,11 +328,17 @@ def latency_sweep(steps, warmup, device):
         ins = [_randn_bf16(P * B, 1.0, 10 + r, device) for r in range(P)]
         outs = [torch.empty(B, dtype=torch.bfloat16, device=device) for _ in range(P)]
         work = [torch.empty_like(t) for t in ins]
+        graph = torch.cuda.CUDAGraph()             # the 7 step launches captured once
+        kernels.reduce_scatter_ranks(outs, ins, "ring", "steps", work)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph):
+            kernels.reduce_scatter_ranks(outs, ins, "ring", "steps", work)
         rows.append({
             "bytes": nbytes,
             "accumulate_us": round(us(lambda: kernels.accumulate(x, y)), 2),
             "copy_us": round(us(lambda: kernels.copy(z, x)), 2),
             "ring_rs_p8_steps_us": round(us(lambda: kernels.reduce_scatter_ranks(outs, ins, "ring", "steps", work)), 2),
+            "ring_rs_p8_steps_graph_us": round(us(graph.replay), 2),
             "ring_rs_p8_fused_us": round(us(lambda: kernels.reduce_scatter_ranks(outs, ins, "ring", "fused")), 2),
         })
     return rows
