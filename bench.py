@@ -333,12 +333,16 @@ def latency_sweep(steps, warmup, device):
         torch.cuda.synchronize()
         with torch.cuda.graph(graph):
             kernels.reduce_scatter_ranks(outs, ins, "ring", "steps", work)
+        plan_fused = kernels.plan_reduce_scatter(outs, ins, "ring", "fused")
+        plan_steps = kernels.plan_reduce_scatter(outs, ins, "ring", "steps", work)
         rows.append({
             "bytes": nbytes,
             "accumulate_us": round(us(lambda: kernels.accumulate(x, y)), 2),
             "copy_us": round(us(lambda: kernels.copy(z, x)), 2),
             "ring_rs_p8_steps_us": round(us(lambda: kernels.reduce_scatter_ranks(outs, ins, "ring", "steps", work)), 2),
             "ring_rs_p8_steps_graph_us": round(us(graph.replay), 2),
+            "ring_rs_p8_steps_plan_us": round(us(plan_steps), 2),
+            "ring_rs_p8_fused_plan_us": round(us(plan_fused), 2),
             "ring_rs_p8_fused_us": round(us(lambda: kernels.reduce_scatter_ranks(outs, ins, "ring", "fused")), 2),
         })
     return rows

@@ -211,6 +211,54 @@ def reduce_scatter_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[torch
                                           B, dtype_code(dt), algorithm, m, stream_handle())
 
 
+class CollectivePlan:
+    """A collective on fixed buffers, validated once: calling the plan only
+    makes the C call (no per-call checks, tables or allocations), which is what
+    a launch-bound small-message loop wants.  The plan keeps its tensors alive."""
+
+    def __init__(self, fn, args, keep):
+        self._fn, self._args, self._keep = fn, args, keep
+
+    def __call__(self):
+        rc = self._fn(*self._args, stream_handle())
+        if rc:
+            raise _native.NativeError(_native.load().last_error())
+
+
+def plan_reduce_scatter(outputs: Sequence[torch.Tensor], inputs: Sequence[torch.Tensor],
+                        algorithm: str = "ring", mode=None,
+                        work: Optional[Sequence[torch.Tensor]] = None) -> CollectivePlan:
+    """Validate like reduce_scatter_ranks, then return a callable that replays
+    the collective on the same buffers."""
+    import ctypes
+    P = len(inputs)
+    m = mode_code(mode)
+    total = inputs[0].numel()
+    if (m == MODE_FAITHFUL and P > 1) or (m == MODE_STEPS and P > 2):
+        if work is None:
+            work = [torch.empty_like(inputs[r]) for r in range(P)]
+    else:
+        work = None
+    # one checked run; raises on any inconsistency
+    reduce_scatter_ranks(outputs, inputs, algorithm, m, work)
+    lib = _native.load()
+    tabs = [_native._ptr_table(_ptrs(outputs)), _native._ptr_table(_ptrs(inputs)), _native._ptr_table(_ptrs(work))]
+    args = (tabs[0], tabs[1], tabs[2], P, total // P, dtype_code(inputs[0].dtype), algorithm.encode(), m)
+    return CollectivePlan(lib._lib.pccl_hip_reduce_scatter_virtual, args,
+                          (list(outputs), list(inputs), None if work is None else list(work), tabs))
+
+
+def plan_all_gather(outputs: Sequence[torch.Tensor], inputs: Sequence[torch.Tensor],
+                    algorithm: str = "recursive", mode=None) -> CollectivePlan:
+    """Validate like all_gather_ranks, then return a callable that replays it."""
+    m = mode_code(mode)
+    all_gather_ranks(outputs, inputs, algorithm, m)
+    lib = _native.load()
+    tabs = [_native._ptr_table(_ptrs(outputs)), _native._ptr_table(_ptrs(inputs))]
+    args = (tabs[0], tabs[1], len(inputs), inputs[0].numel() * inputs[0].element_size(), algorithm.encode(), m)
+    return CollectivePlan(lib._lib.pccl_hip_all_gather_virtual, args, (list(outputs), list(inputs), tabs))
+
+
 def all_gather_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[torch.Tensor],
                      algorithm: str = "recursive", mode=None) -> None:
     """all_gather over P virtual ranks: outputs[r] = cat(inputs) for every r

@@ -356,6 +356,30 @@ def test_2d_per_rank_api_with_two_grids(target, mode, monkeypatch):
             assert_bits_equal(to_numpy(g_out[g * per + k], O.BF16), np.concatenate(want), f"gather grid {g} rank {k}")
 
 
+@pytest.mark.parametrize("mode", MODES)
+def test_plans_replay_on_fresh_data(target, mode):
+    """A validated plan replays the collective with no per-call checks."""
+    import torch
+    from pccl import kernels
+    P, B, dtype = 4, 515, O.F32
+    ins = make_inputs(P, P * B, dtype, seed=91)
+    t_in = [to_torch(x, dtype, target.device) for x in ins]
+    t_out = [torch.zeros(B, device=target.device) for _ in range(P)]
+    plan = kernels.plan_reduce_scatter(t_out, t_in, "ring", mode)
+    g_out = [torch.zeros(P * B, device=target.device) for _ in range(P)]
+    gplan = kernels.plan_all_gather(g_out, t_out, "ring", mode)
+    fresh = make_inputs(P, P * B, dtype, seed=92)
+    for t, x in zip(t_in, fresh):
+        t.copy_(to_torch(x, dtype, target.device))
+    plan()
+    gplan()
+    target.sync()
+    want = O.ring_reduce_scatter(fresh, dtype)
+    for r in range(P):
+        assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"rank {r}")
+        assert_bits_equal(to_numpy(g_out[r], dtype), np.concatenate(want), f"gather rank {r}")
+
+
 @pytest.mark.parametrize("rec", [True, False])
 def test_all_reduce(target, rec):
     import torch
