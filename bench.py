@@ -15,6 +15,8 @@ Workloads (`cfg2` is the one the headline metric is quoted on):
         accumulate with bf16 rounding at every hop              (default)
   cfg3  recursive-halving round at its largest shape: a pair of ranks adding
         512 MiB strided halves (bf16), i.e. round 0 of P=64 with 1 GiB per rank
+  cfg3full  the whole recursive-halving reduce_scatter over P=64 resident ranks,
+        bf16, 1 GiB per rank (64 GiB of inputs + 64 GiB of work buffers in HBM)
   cfg4  all_gather placement, P=16, bf16 shards of 128 MiB into 2 GiB outputs
   cfg4u the same with uneven shards padded to 256 bytes
   cfg5  fused one-pass reduce of 32 fp32 shards of 32 Mi elements
@@ -52,7 +54,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg2",
-                    choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg4u", "cfg5", "latency", "ceilings"])
+                    choices=["cfg1", "cfg2", "cfg3", "cfg3full", "cfg4", "cfg4u", "cfg5", "latency", "ceilings"])
     ap.add_argument("--mode", default=None, choices=["steps", "fused", "faithful"],
                     help="execution mode of the collective (default: per-step replay)")
     ap.add_argument("--scale", type=float, default=1.0,
@@ -172,6 +174,49 @@ def make_rh_pair(count_elems, device, seed=7):
     return step, info
 
 
+def make_rh_full(P, elems_per_rank, mode, device, seed=21):
+    """Recursive-halving reduce_scatter with all P ranks resident."""
+    import torch
+    from pccl import kernels
+    B = elems_per_rank // P
+    total = B * P
+    ins = [_randn_bf16(total, 1.0, seed + r, device) for r in range(P)]
+    outs = [torch.empty(B, dtype=torch.bfloat16, device=device) for _ in range(P)]
+    m = kernels.mode_code(mode)
+    work = [torch.empty_like(ins[r]) for r in range(P)] if m != kernels.MODE_FUSED else None
+
+    def step():
+        kernels.reduce_scatter_ranks(outs, ins, "recursive", m, work)
+
+    def verify():
+        # the halving order of block 0 and block P-1 recomputed with torch on a window
+        n = min(B, 1 << 20)
+        for j in (0, P - 1):
+            v = [ins[j ^ q][j * B:j * B + n].float() for q in range(P)]
+            h = P // 2
+            while h >= 1:
+                for q in range(h):
+                    v[q] = (v[q] + v[q + h]).bfloat16().float()
+                h //= 2
+            if not torch.equal(outs[j][:n].float(), v[0]):
+                return False
+        return True
+
+    rounds = P.bit_length() - 1
+    if m == kernels.MODE_FUSED:
+        kb = (P * P + P) * B * 2
+        alg, kernel, kl, launches = kb, "k_reduce_kway", 1, 1
+    else:
+        # round r adds (P / 2^(r+1)) blocks per rank: 2 reads + 1 write per element
+        alg = sum(3 * P * (P >> (r + 1)) * B * 2 for r in range(rounds))
+        kb, kernel, kl, launches = alg, "k_rh_round", 1, rounds
+    info = dict(alg_bytes=alg, kernel=kernel, kernel_bytes=kb, kernel_launches=kl, launches=launches,
+                desc=f"recursive-halving reduce_scatter, P={P} resident virtual ranks, bf16, {total} elements per "
+                     f"rank ({total * 2 / MiB:.0f} MiB), {rounds} rounds, mode={_mode_name(m)}",
+                dtype="bf16", P=P, B=B, verify=verify)
+    return step, info
+
+
 def make_all_gather(P, shard_bytes, mode, device, uneven=False, seed=3):
     import torch
     from pccl import kernels
@@ -258,6 +303,8 @@ def build_workload(name, mode, scale, device):
         return make_ring_rs(8, sc(256 * MiB), "bf16", mode, device, std=1e-2)
     if name == "cfg3":
         return make_rh_pair(sc(256 * MiB), device)
+    if name == "cfg3full":
+        return make_rh_full(64, sc(512 * MiB, 1 << 16), mode, device)
     if name == "cfg4":
         return make_all_gather(16, sc(128 * MiB), mode, device)
     if name == "cfg4u":
@@ -485,6 +532,9 @@ def main():
     # faithful mode, the copies), so its mean launch time is region / launches
     if info["launches"] == info["kernel_launches"]:
         kernel_ms = dev_ms / (args.steps * info["kernel_launches"])
+    elif info["kernel_bytes"] == info["alg_bytes"]:
+        # launches of different sizes (halving rounds): bytes and time of the whole sequence
+        kernel_ms = dev_ms / args.steps
     else:
         kernel_ms = None
     roof = None
