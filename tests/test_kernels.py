@@ -255,3 +255,40 @@ def test_probe_streams(target):
     from pccl._native import NativeError
     with pytest.raises(NativeError, match="kind must be"):
         target.native.probe_stream(2, buf.data_ptr(), n * 4, target.stream())
+
+
+@pytest.mark.parametrize("unroll", [1, 2, 4, 8])
+@pytest.mark.parametrize("nt", [0, 1])
+@pytest.mark.parametrize("grid_cap", [0, 3, 64])
+def test_every_launch_tuning_gives_the_same_bits(target, unroll, nt, grid_cap):
+    """Unroll depth, non-temporal hints and a capped (grid-stride) launch change
+    speed only."""
+    import torch
+    from pccl import kernels
+    lib = target.native
+    saved = {k: lib.get_tuning(k) for k in ("unroll", "nt_load", "nt_store", "grid_cap")}
+    try:
+        lib.set_tuning("unroll", unroll)
+        lib.set_tuning("nt_load", nt)
+        lib.set_tuning("nt_store", nt)
+        lib.set_tuning("grid_cap", grid_cap)
+        P, B = 4, 9001
+        for dtype in DTYPES:
+            ins = make_inputs(P, P * B, dtype, seed=17)
+            t_in = [to_torch(x, dtype, target.device) for x in ins]
+            for alg, ref in (("ring", O.ring_reduce_scatter), ("recursive", O.recursive_halving_reduce_scatter)):
+                want = ref(ins, dtype)
+                for mode in ("steps", "fused", "faithful"):
+                    t_out = [torch.zeros(B, dtype=t_in[0].dtype, device=target.device) for _ in range(P)]
+                    kernels.reduce_scatter_ranks(t_out, t_in, alg, mode)
+                    target.sync()
+                    for r in range(P):
+                        assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"{alg}/{mode}/{dtype} rank {r}")
+            g_out = [torch.zeros(P * P * B, dtype=t_in[0].dtype, device=target.device) for _ in range(P)]
+            for mode in ("steps", "fused"):
+                kernels.all_gather_ranks(g_out, t_in, "recursive", mode)
+                target.sync()
+                assert_bits_equal(to_numpy(g_out[P - 1], dtype), np.concatenate(ins), f"all_gather {mode}")
+    finally:
+        for k, v in saved.items():
+            lib.set_tuning(k, v)
