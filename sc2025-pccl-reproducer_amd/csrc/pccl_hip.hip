@@ -61,6 +61,16 @@ using namespace pccl_kernels;
 // ---------------------------------------------------------------------------
 // host side: launch geometry and dispatch over the tuning parameters
 // ---------------------------------------------------------------------------
+// Kernels count their work items (tiles) in 32 bits.
+constexpr size_t kMaxWorkItems = 0xffffffffull;
+
+int check_work_items(size_t segments, size_t tiles, const char* what) {
+  if (tiles != 0 && segments > kMaxWorkItems / tiles)
+    return fail(PCCL_HIP_EINVAL, "%s: %zu segments of %zu tiles exceed the 2^32 - 1 tiles of one launch", what,
+                segments, tiles);
+  return PCCL_HIP_OK;
+}
+
 unsigned grid_for(size_t total_tiles) {
   long cap = g_grid_cap.load(std::memory_order_relaxed);
   size_t g = total_tiles;
@@ -145,6 +155,7 @@ int launch_add_pieces(const AddSegs& segs, int count, const Pieces& pc, int dtyp
   if (pc.len == 0 || count == 0 || pc.s1 == 0 || pc.s2 == 0) return PCCL_HIP_OK;
   Tune t = current_tune();
   AddLaunch l{&segs, count, dtype, pc, tiles_for(pc.len * esize_of(dtype), t.unroll), stream};
+  if (int rc = check_work_items((size_t)count * pc.s1 * pc.s2, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);
 }
@@ -172,6 +183,7 @@ int launch_copy(const CopySegs& segs, int count, hipStream_t stream, const char*
   if (longest == 0 || count == 0) return PCCL_HIP_OK;
   Tune t = current_tune();
   CopyLaunch l{&segs, count, tiles_for(longest, t.unroll), stream};
+  if (int rc = check_work_items((size_t)count, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);
 }
@@ -194,6 +206,7 @@ int launch_copy_pieces(const CopyPairs& segs, int count, const Pieces& pc, hipSt
   if (pc.len == 0 || count == 0 || pc.s1 == 0 || pc.s2 == 0) return PCCL_HIP_OK;
   Tune t = current_tune();
   CopyPiecesLaunch l{&segs, count, pc, tiles_for(pc.len, t.unroll), stream};
+  if (int rc = check_work_items((size_t)count * pc.s1 * pc.s2, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);
 }
@@ -248,12 +261,12 @@ struct TransposeLaunch {
 struct KwayLaunch {
   const KwayArgs* args;
   int k, g, nout, dtype, order, first0, per_hop;
-  size_t n;
+  size_t n, tiles;
   hipStream_t stream;
 
   template <class Acc, int U, bool NTL, bool NTS>
   void run() const {
-    size_t tiles = tiles_for(n * sizeof(typename Acc::op::elem), U);
+    static_assert(U == 1, "the fused reduce is launched with one vector per thread");
     unsigned grid = grid_for((size_t)nout * tiles);
 #define PCCL_KWAY(KV) \
   hipLaunchKernelGGL((k_reduce_kway<Acc, KV, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *args, k, g, nout, n, first0, tiles)
@@ -282,7 +295,8 @@ struct KwayLaunch {
 int launch_kway(const KwayArgs& args, int k, int g, int nout, size_t n, int dtype, int order,
                 int first0, int per_hop, hipStream_t stream, const char* what) {
   if (n == 0 || nout == 0) return PCCL_HIP_OK;
-  KwayLaunch l{&args, k, g, nout, dtype, order, first0, per_hop, n, stream};
+  KwayLaunch l{&args, k, g, nout, dtype, order, first0, per_hop, n, tiles_for(n * esize_of(dtype), 1), stream};
+  if (int rc = check_work_items((size_t)nout, l.tiles, what)) return rc;
   with_tuning(current_tune(), l);
   return launch_status(what);
 }
@@ -406,6 +420,7 @@ int pccl_hip_rh_round(void* const* bufs, const void* const* src, void* const* ou
   Tune t = current_tune();
   RhLaunch l{&args, P, round, dtype, src ? 1 : 0, to_outs ? 1 : 0, B,
              tiles_for(count * esize_of(dtype), t.unroll), (hipStream_t)stream};
+  if (int rc = check_work_items((size_t)P, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);
 }
@@ -468,6 +483,9 @@ int pccl_hip_block_transpose(void* dst, const void* src, size_t rows, size_t col
   Tune t = current_tune();
   TransposeLaunch l{(uint8_t*)dst, (const uint8_t*)src, rows, cols, m_bytes,
                     tiles_for(m_bytes, t.unroll), (hipStream_t)stream};
+  if (rows > kMaxWorkItems || cols > kMaxWorkItems / rows)
+    return fail(PCCL_HIP_EINVAL, "%s: rows*cols too large", what);
+  if (int rc = check_work_items(rows * cols, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);
 }
@@ -491,6 +509,7 @@ int pccl_hip_all_gather_uneven_virtual(void* const* outputs, const void* const* 
   if (longest == 0) return PCCL_HIP_OK;
   Tune t = current_tune();
   GatherLaunch l{&args, P, P, tiles_for(longest, t.unroll), (hipStream_t)stream};
+  if (int rc = check_work_items((size_t)P, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);
 }

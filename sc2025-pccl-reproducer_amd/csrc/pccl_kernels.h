@@ -319,14 +319,17 @@ template <class Op, int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_add_segs(AddSegs t, int count, Pieces pc,
                                                        size_t tiles_per_piece) {
   typedef typename Op::elem elem;
-  const size_t per_seg = (size_t)pc.s1 * pc.s2 * tiles_per_piece;
-  const size_t total = (size_t)count * per_seg;
-  for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
-    const int s = (int)(w / per_seg);
-    const size_t rem = w - (size_t)s * per_seg;
-    const size_t piece = rem / tiles_per_piece;
-    const size_t tile = rem - piece * tiles_per_piece;
-    const size_t p1 = piece / pc.s2, p2 = piece - p1 * pc.s2;
+  // work items are counted in 32 bits (the host refuses launches beyond 2^32 - 1)
+  const uint32_t tpp = (uint32_t)tiles_per_piece;
+  const uint32_t per_seg = pc.s1 * pc.s2 * tpp;
+  const uint64_t total = (uint64_t)count * per_seg;
+  for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
+    const uint32_t w = (uint32_t)w64;
+    const uint32_t s = w / per_seg;
+    const uint32_t rem = w - s * per_seg;
+    const uint32_t piece = rem / tpp;
+    const size_t tile = rem - piece * tpp;
+    const size_t p1 = piece / pc.s2, p2 = piece - (uint32_t)p1 * pc.s2;
     add_tile<Op, U, NTL, NTS>((elem*)t.dst[s] + p1 * pc.d1 + p2 * pc.d2,
                               (const elem*)t.a[s] + p1 * pc.a1 + p2 * pc.a2,
                               (const elem*)t.b[s] + p1 * pc.b1 + p2 * pc.b2, pc.len, tile);
@@ -351,10 +354,12 @@ __global__ __launch_bounds__(kThreads) void k_rh_round(RhArgs t, int P, size_t B
   const int group = P >> round;
   const int half = group >> 1;
   const size_t count = (size_t)half * B;
-  const size_t total = (size_t)P * tiles_per_seg;
-  for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
-    const int r = (int)(w / tiles_per_seg);
-    const size_t tile = w - (size_t)r * tiles_per_seg;
+  const uint32_t tps = (uint32_t)tiles_per_seg;
+  const uint64_t total = (uint64_t)P * tps;
+  for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
+    const uint32_t w = (uint32_t)w64;
+    const int r = (int)(w / tps);
+    const size_t tile = w - (uint32_t)r * tps;
     const bool lower = (r % group) < half;
     const int partner = lower ? r + half : r - half;
     const size_t off = (size_t)(r / group) * group * B + (lower ? 0 : count);
@@ -375,11 +380,13 @@ struct CopySegs {
 template <int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_copy_segs(CopySegs t, int count,
                                                         size_t tiles_per_seg) {
-  const size_t total = (size_t)count * tiles_per_seg;
+  const uint32_t tps = (uint32_t)tiles_per_seg;
+  const uint64_t total = (uint64_t)count * tps;
   const size_t tile_bytes = (size_t)kThreads * U * 16;
-  for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
-    const int s = (int)(w / tiles_per_seg);
-    const size_t tile = w - (size_t)s * tiles_per_seg;
+  for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
+    const uint32_t w = (uint32_t)w64;
+    const int s = (int)(w / tps);
+    const size_t tile = w - (uint32_t)s * tps;
     const size_t nb = t.nbytes[s];
     // a tile past the end of a short segment has nothing to do (16 spare
     // bytes cover the head shift of the vector body)
@@ -397,14 +404,17 @@ struct CopyPairs {
 template <int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_copy_pieces(CopyPairs t, int count, Pieces pc,
                                                           size_t tiles_per_piece) {
-  const size_t per_seg = (size_t)pc.s1 * pc.s2 * tiles_per_piece;
-  const size_t total = (size_t)count * per_seg;
-  for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
-    const int s = (int)(w / per_seg);
-    const size_t rem = w - (size_t)s * per_seg;
-    const size_t piece = rem / tiles_per_piece;
-    const size_t tile = rem - piece * tiles_per_piece;
-    const size_t p1 = piece / pc.s2, p2 = piece - p1 * pc.s2;
+  // work items are counted in 32 bits (the host refuses launches beyond 2^32 - 1)
+  const uint32_t tpp = (uint32_t)tiles_per_piece;
+  const uint32_t per_seg = pc.s1 * pc.s2 * tpp;
+  const uint64_t total = (uint64_t)count * per_seg;
+  for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
+    const uint32_t w = (uint32_t)w64;
+    const uint32_t s = w / per_seg;
+    const uint32_t rem = w - s * per_seg;
+    const uint32_t piece = rem / tpp;
+    const size_t tile = rem - piece * tpp;
+    const size_t p1 = piece / pc.s2, p2 = piece - (uint32_t)p1 * pc.s2;
     copy_tile<U, NTL, NTS>((uint8_t*)t.dst[s] + p1 * pc.d1 + p2 * pc.d2,
                            (const uint8_t*)t.src[s] + p1 * pc.a1 + p2 * pc.a2, pc.len, tile);
   }
@@ -423,12 +433,14 @@ struct GatherArgs {
 template <int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_gather_multicast(GatherArgs t, int P, int nout,
                                                               size_t tiles_per_seg) {
-  const size_t total = (size_t)P * tiles_per_seg;
+  const uint32_t tps = (uint32_t)tiles_per_seg;
+  const uint64_t total = (uint64_t)P * tps;
   const size_t tile_bytes = (size_t)kThreads * U * 16;
   const unsigned tid = threadIdx.x;
-  for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
-    const int k = (int)(w / tiles_per_seg);
-    const size_t tile = w - (size_t)k * tiles_per_seg;
+  for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
+    const uint32_t w = (uint32_t)w64;
+    const int k = (int)(w / tps);
+    const size_t tile = w - (uint32_t)k * tps;
     const size_t nb = t.nbytes[k];
     if (tile != 0 && tile * tile_bytes >= nb + 16) continue;
     const uint8_t* src = (const uint8_t*)t.ins[k];
@@ -464,11 +476,14 @@ template <int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_block_transpose(uint8_t* dst, const uint8_t* src,
                                                               size_t rows, size_t cols, size_t m,
                                                               size_t tiles_per_seg) {
-  const size_t total = rows * cols * tiles_per_seg;
-  for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
-    const size_t blk = w / tiles_per_seg;            // destination block index c*rows + r
-    const size_t tile = w - blk * tiles_per_seg;
-    const size_t c = blk / rows, r = blk - c * rows;
+  const uint32_t tps = (uint32_t)tiles_per_seg;
+  const uint64_t total = (uint64_t)rows * cols * tps;
+  for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
+    const uint32_t w = (uint32_t)w64;
+    const uint32_t blk32 = w / tps;                  // destination block index c*rows + r
+    const size_t tile = w - blk32 * tps;
+    const size_t blk = blk32;
+    const size_t c = blk32 / (uint32_t)rows, r = blk - c * rows;
     copy_tile<U, NTL, NTS>(dst + blk * m, src + (r * cols + c) * m, m, tile);
   }
 }
@@ -602,11 +617,13 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
   typedef typename Acc::op Op;
   typedef typename Op::elem elem;
   constexpr int L = Acc::kLanes;
-  const size_t total = (size_t)nout * tiles_per_seg;
+  const uint32_t tps = (uint32_t)tiles_per_seg;
+  const uint64_t total = (uint64_t)nout * tps;
   const unsigned tid = threadIdx.x;
-  for (size_t w = blockIdx.x; w < total; w += gridDim.x) {
-    const int j = (int)(w / tiles_per_seg);
-    const size_t tile = w - (size_t)j * tiles_per_seg;
+  for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
+    const uint32_t w = (uint32_t)w64;
+    const int j = (int)(w / tps);
+    const size_t tile = w - (uint32_t)j * tps;
     // flat: the schedule of output j starts at shard (first0 + j) mod k;
     // two-level ring (g < k): inner start (j mod g) + 1, outer start (j / g) + 1
     const int first = g >= k ? (first0 + j) % k : (j % g + 1) % g;
