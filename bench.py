@@ -22,6 +22,8 @@ Workloads (`cfg2` is the one the headline metric is quoted on):
   cfg5  fused one-pass reduce of 32 fp32 shards of 32 Mi elements
   ceilings  what the device sustains for plain streams of 1 GiB: read-only,
         write-only, copy and 2-reads-1-write add (the practical roofline)
+  sweep  GB/s against message size, 64 MiB .. 2 GiB per operand: accumulate
+        (bf16 and fp32), copy, and the fused 8-way reduce
   latency  small messages, 4 KiB .. 1 MiB in bf16: microseconds per accumulate,
         per copy and per whole P=8 ring reduce_scatter (per-step and fused)
 
@@ -54,7 +56,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg2",
-                    choices=["cfg1", "cfg2", "cfg3", "cfg3full", "cfg4", "cfg4u", "cfg5", "latency", "ceilings"])
+                    choices=["cfg1", "cfg2", "cfg3", "cfg3full", "cfg4", "cfg4u", "cfg5", "latency", "ceilings", "sweep"])
     ap.add_argument("--mode", default=None, choices=["steps", "fused", "faithful"],
                     help="execution mode of the collective (default: per-step replay)")
     ap.add_argument("--scale", type=float, default=1.0,
@@ -348,6 +350,43 @@ def ceilings(steps, warmup, device):
     }
 
 
+def size_sweep(steps, warmup, device):
+    """Achieved GB/s of the per-hop, copy and fused kernels against message size."""
+    import torch
+    from pccl import kernels
+
+    def gbps(fn, nbytes):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(steps):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return round(nbytes / (s.elapsed_time(e) / steps * 1e-3) / 1e9, 1)
+
+    rows = []
+    for mib in (64, 128, 256, 512, 1024, 2048):
+        nb = mib * MiB
+        a16, b16 = _randn_bf16(nb // 2, 1e-2, 1, device), _randn_bf16(nb // 2, 1e-2, 2, device)
+        a32, b32 = a16.view(torch.float32), b16.view(torch.float32)
+        c = torch.empty_like(a16)
+        k = 8
+        shards = [_randn_bf16(nb // 2 // k, 1e-2, 10 + i, device) for i in range(k)]
+        out = torch.empty_like(shards[0])
+        rows.append({
+            "MiB": mib,
+            "accumulate_bf16": gbps(lambda: kernels.accumulate(a16, b16), 3 * nb),
+            "accumulate_f32": gbps(lambda: kernels.accumulate(a32, b32), 3 * nb),
+            "copy": gbps(lambda: kernels.copy(c, a16), 2 * nb),
+            "reduce_8way_bf16_total_input": gbps(lambda: kernels.reduce_kway(out, shards, "ring", 1), (k + 1) * nb // k),
+        })
+        del a16, b16, a32, b32, c, shards, out
+    return rows
+
+
 def latency_sweep(steps, warmup, device):
     """Microseconds per call for launch-bound message sizes (bf16)."""
     import torch
@@ -480,6 +519,20 @@ def main():
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
             "config": {"workload": "ceilings: plain streams over 1 GiB buffers; value = the library's add kernel",
                        "GBps": res}, "roofline": None, "cpu_baseline": None}), flush=True)
+        return 0
+
+    if args.workload == "sweep":
+        rows = size_sweep(args.steps, args.warmup, device)
+        big = [r for r in rows if r["MiB"] >= 256]
+        val = round(sum(r["accumulate_bf16"] for r in big) / len(big), 1)
+        print(json.dumps({
+            "metric": METRIC, "value": val, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+            "data": "synthetic",
+            "config": {"workload": "sweep: GB/s against message size (MiB per operand); value = mean accumulate "
+                                   "bf16 at >= 256 MiB", "GBps": rows,
+                       "pct_of_hbm_peak": round(100 * val / HBM_PEAK_GBPS, 2)},
+            "roofline": None, "cpu_baseline": None}), flush=True)
         return 0
 
     if args.workload == "latency":
