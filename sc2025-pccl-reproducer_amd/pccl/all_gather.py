@@ -32,6 +32,7 @@ def recursive_doubling_allgather_mpi(output_tensor: torch.Tensor,
     rank, size = comm.Get_rank(), comm.Get_size()
     block_size = input_tensor.numel()
     assert output_tensor.numel() == size * block_size, "Output tensor has incorrect size"
+    assert size & (size - 1) == 0, "recursive doubling needs a power-of-two number of processes"
     kernels.check_device_tensor(input_tensor, "input")
     kernels.check_device_tensor(output_tensor, "output")
 

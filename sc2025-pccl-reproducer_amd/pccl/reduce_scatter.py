@@ -65,6 +65,8 @@ def recursive_halving_reduce_scatter_mpi(output_tensor: torch.Tensor,
     total_elems = input_tensor.numel()
     assert total_elems % size == 0, "Input tensor size must be divisible by number of processes"
     block_size = total_elems // size
+    # the reference silently assumes a power of two (int(log2 P) rounds); fail instead of mis-reducing
+    assert size & (size - 1) == 0, "recursive halving needs a power-of-two number of processes"
     kernels.check_device_tensor(input_tensor, "input")
     kernels.check_device_tensor(output_tensor, "output")
 
