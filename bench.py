@@ -67,7 +67,7 @@ def parse_args():
                     help="after the timed region launch one plain 1 GiB device copy (k_copy_segs): its "
                          "FETCH_SIZE / WRITE_SIZE readings scale the hardware counters of a rocprofv3 --pmc run")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
-                    help="launch tuning of the library (grid_cap, unroll, nt_load, nt_store)")
+                    help="launch tuning of the library (grid_cap, unroll, unroll_copy, nt_load, nt_store)")
     return ap.parse_args()
 
 
@@ -614,7 +614,7 @@ def main():
         "config": {"workload": f"{args.workload}: {info['desc']}", "algorithmic_bytes_per_step": info["alg_bytes"],
                    "launches_per_step": info["launches"], "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
                    "wall_ms_per_step": round(wall_ms / args.steps, 4), "verified": ok,
-                   "tuning": {k: lib.get_tuning(k) for k in ("grid_cap", "unroll", "nt_load", "nt_store")}},
+                   "tuning": {k: lib.get_tuning(k) for k in ("grid_cap", "unroll", "unroll_copy", "nt_load", "nt_store")}},
         "roofline": roof, "cpu_baseline": cpu,
     }
     print(json.dumps(out), flush=True)

@@ -46,7 +46,8 @@ int launch_status(const char* what) {
 }
 
 std::atomic<long> g_grid_cap{0};
-std::atomic<long> g_unroll{4};
+std::atomic<long> g_unroll{4};        // vectors per thread and operand, add kernels
+std::atomic<long> g_unroll_copy{2};   // ... copy kernels (8 KiB per workgroup: best across 64 MiB - 2 GiB)
 std::atomic<long> g_nt_load{1};
 std::atomic<long> g_nt_store{1};
 
@@ -92,9 +93,11 @@ struct Tune {
   bool ntl, nts;
 };
 
-Tune current_tune() {
+bool is16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+Tune current_tune(bool copy = false) {
   Tune t;
-  t.unroll = (int)g_unroll.load(std::memory_order_relaxed);
+  t.unroll = (int)(copy ? g_unroll_copy : g_unroll).load(std::memory_order_relaxed);
   t.ntl = g_nt_load.load(std::memory_order_relaxed) != 0;
   t.nts = g_nt_store.load(std::memory_order_relaxed) != 0;
   return t;
@@ -139,22 +142,34 @@ struct AddLaunch {
   int count, dtype;
   Pieces pc;
   size_t tiles;
+  int aligned;
   hipStream_t stream;
   template <int U, bool NTL, bool NTS>
   void operator()() const {
     unsigned grid = grid_for((size_t)count * pc.s1 * pc.s2 * tiles);
     if (dtype == PCCL_HIP_F32)
-      hipLaunchKernelGGL((k_add_segs<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, pc, tiles);
+      hipLaunchKernelGGL((k_add_segs<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, pc, tiles, aligned);
     else
-      hipLaunchKernelGGL((k_add_segs<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, pc, tiles);
+      hipLaunchKernelGGL((k_add_segs<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, pc, tiles, aligned);
   }
 };
+
+// True if every piece of every operand starts on a 16-byte boundary and is a
+// whole number of vectors: the kernels then skip all head/tail handling.
+bool pieces_aligned(const Pieces& pc, size_t unit) {
+  const size_t m = 16 / unit - 1;   // strides and length are in units of `unit` bytes
+  auto ok = [&](size_t v) { return (v & m) == 0; };
+  return ok(pc.len) && (pc.s1 < 2 || (ok(pc.d1) && ok(pc.a1) && ok(pc.b1))) &&
+         (pc.s2 < 2 || (ok(pc.d2) && ok(pc.a2) && ok(pc.b2)));
+}
 
 int launch_add_pieces(const AddSegs& segs, int count, const Pieces& pc, int dtype, hipStream_t stream,
                       const char* what) {
   if (pc.len == 0 || count == 0 || pc.s1 == 0 || pc.s2 == 0) return PCCL_HIP_OK;
   Tune t = current_tune();
-  AddLaunch l{&segs, count, dtype, pc, tiles_for(pc.len * esize_of(dtype), t.unroll), stream};
+  bool aligned = pieces_aligned(pc, esize_of(dtype));
+  for (int s = 0; s < count && aligned; ++s) aligned = is16(segs.dst[s]) && is16(segs.a[s]) && is16(segs.b[s]);
+  AddLaunch l{&segs, count, dtype, pc, tiles_for(pc.len * esize_of(dtype), t.unroll), aligned ? 1 : 0, stream};
   if (int rc = check_work_items((size_t)count * pc.s1 * pc.s2, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);
@@ -169,11 +184,12 @@ struct CopyLaunch {
   const CopySegs* segs;
   int count;
   size_t tiles;
+  int aligned;
   hipStream_t stream;
   template <int U, bool NTL, bool NTS>
   void operator()() const {
     unsigned grid = grid_for((size_t)count * tiles);
-    hipLaunchKernelGGL((k_copy_segs<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, tiles);
+    hipLaunchKernelGGL((k_copy_segs<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, tiles, aligned);
   }
 };
 
@@ -181,8 +197,11 @@ int launch_copy(const CopySegs& segs, int count, hipStream_t stream, const char*
   size_t longest = 0;
   for (int s = 0; s < count; ++s) longest = segs.nbytes[s] > longest ? segs.nbytes[s] : longest;
   if (longest == 0 || count == 0) return PCCL_HIP_OK;
-  Tune t = current_tune();
-  CopyLaunch l{&segs, count, tiles_for(longest, t.unroll), stream};
+  Tune t = current_tune(true);
+  bool aligned = true;
+  for (int s = 0; s < count && aligned; ++s)
+    aligned = segs.nbytes[s] == 0 || (is16(segs.dst[s]) && is16(segs.src[s]) && (segs.nbytes[s] & 15u) == 0);
+  CopyLaunch l{&segs, count, tiles_for(longest, t.unroll), aligned ? 1 : 0, stream};
   if (int rc = check_work_items((size_t)count, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);
@@ -193,19 +212,24 @@ struct CopyPiecesLaunch {
   int count;
   Pieces pc;
   size_t tiles;
+  int aligned;
   hipStream_t stream;
   template <int U, bool NTL, bool NTS>
   void operator()() const {
     unsigned grid = grid_for((size_t)count * pc.s1 * pc.s2 * tiles);
-    hipLaunchKernelGGL((k_copy_pieces<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, pc, tiles);
+    hipLaunchKernelGGL((k_copy_pieces<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, pc, tiles, aligned);
   }
 };
 
 int launch_copy_pieces(const CopyPairs& segs, int count, const Pieces& pc, hipStream_t stream,
                        const char* what) {
   if (pc.len == 0 || count == 0 || pc.s1 == 0 || pc.s2 == 0) return PCCL_HIP_OK;
-  Tune t = current_tune();
-  CopyPiecesLaunch l{&segs, count, pc, tiles_for(pc.len, t.unroll), stream};
+  Tune t = current_tune(true);
+  Pieces chk = pc;
+  chk.b1 = chk.b2 = 0;
+  bool aligned = pieces_aligned(chk, 1);
+  for (int s = 0; s < count && aligned; ++s) aligned = is16(segs.dst[s]) && is16(segs.src[s]);
+  CopyPiecesLaunch l{&segs, count, pc, tiles_for(pc.len, t.unroll), aligned ? 1 : 0, stream};
   if (int rc = check_work_items((size_t)count * pc.s1 * pc.s2, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);
@@ -215,16 +239,17 @@ struct RhLaunch {
   const RhArgs* args;
   int P, round, dtype, from_src, to_outs;
   size_t B, tiles;
+  int aligned;
   hipStream_t stream;
   template <int U, bool NTL, bool NTS>
   void operator()() const {
     unsigned grid = grid_for((size_t)P * tiles);
     if (dtype == PCCL_HIP_F32)
       hipLaunchKernelGGL((k_rh_round<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *args, P, B, round, from_src,
-                                                                    to_outs, tiles);
+                                                                    to_outs, tiles, aligned);
     else
       hipLaunchKernelGGL((k_rh_round<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *args, P, B, round, from_src,
-                                                                     to_outs, tiles);
+                                                                     to_outs, tiles, aligned);
   }
 };
 
@@ -247,11 +272,12 @@ struct TransposeLaunch {
   uint8_t* dst;
   const uint8_t* src;
   size_t rows, cols, m, tiles;
+  int aligned;
   hipStream_t stream;
   template <int U, bool NTL, bool NTS>
   void operator()() const {
     unsigned grid = grid_for(rows * cols * tiles);
-    hipLaunchKernelGGL((k_block_transpose<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, dst, src, rows, cols, m, tiles);
+    hipLaunchKernelGGL((k_block_transpose<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, dst, src, rows, cols, m, tiles, aligned);
   }
 };
 
@@ -338,6 +364,10 @@ int pccl_hip_set_tuning(const char* key, long value) {
     if (value != 1 && value != 2 && value != 4 && value != 8)
       return fail(PCCL_HIP_EINVAL, "set_tuning: unroll must be 1, 2, 4 or 8");
     g_unroll = value;
+  } else if (!strcmp(key, "unroll_copy")) {
+    if (value != 1 && value != 2 && value != 4 && value != 8)
+      return fail(PCCL_HIP_EINVAL, "set_tuning: unroll_copy must be 1, 2, 4 or 8");
+    g_unroll_copy = value;
   } else if (!strcmp(key, "nt_load")) {
     g_nt_load = value != 0;
   } else if (!strcmp(key, "nt_store")) {
@@ -352,6 +382,7 @@ long pccl_hip_get_tuning(const char* key) {
   if (!key) return -1;
   if (!strcmp(key, "grid_cap")) return g_grid_cap;
   if (!strcmp(key, "unroll")) return g_unroll;
+  if (!strcmp(key, "unroll_copy")) return g_unroll_copy;
   if (!strcmp(key, "nt_load")) return g_nt_load;
   if (!strcmp(key, "nt_store")) return g_nt_store;
   return -1;
@@ -418,8 +449,12 @@ int pccl_hip_rh_round(void* const* bufs, const void* const* src, void* const* ou
   }
   const size_t count = (size_t)((P >> round) / 2) * B;
   Tune t = current_tune();
+  // block offsets are multiples of B elements, so B must be a whole number of vectors too
+  bool aligned = (B * esize_of(dtype)) % 16 == 0;
+  for (int r = 0; r < P && aligned; ++r)
+    aligned = is16(args.bufs[r]) && is16(args.src[r]) && is16(args.outs[r]);
   RhLaunch l{&args, P, round, dtype, src ? 1 : 0, to_outs ? 1 : 0, B,
-             tiles_for(count * esize_of(dtype), t.unroll), (hipStream_t)stream};
+             tiles_for(count * esize_of(dtype), t.unroll), aligned ? 1 : 0, (hipStream_t)stream};
   if (int rc = check_work_items((size_t)P, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);
@@ -480,9 +515,10 @@ int pccl_hip_block_transpose(void* dst, const void* src, size_t rows, size_t col
   const char* what = "pccl_hip_block_transpose";
   if (rows == 0 || cols == 0 || m_bytes == 0) return PCCL_HIP_OK;
   if (!dst || !src) return fail(PCCL_HIP_EINVAL, "%s: NULL operand", what);
-  Tune t = current_tune();
+  Tune t = current_tune(true);
+  const bool aligned = is16(dst) && is16(src) && (m_bytes & 15u) == 0;
   TransposeLaunch l{(uint8_t*)dst, (const uint8_t*)src, rows, cols, m_bytes,
-                    tiles_for(m_bytes, t.unroll), (hipStream_t)stream};
+                    tiles_for(m_bytes, t.unroll), aligned ? 1 : 0, (hipStream_t)stream};
   if (rows > kMaxWorkItems || cols > kMaxWorkItems / rows)
     return fail(PCCL_HIP_EINVAL, "%s: rows*cols too large", what);
   if (int rc = check_work_items(rows * cols, l.tiles, what)) return rc;

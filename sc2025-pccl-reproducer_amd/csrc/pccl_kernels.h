@@ -188,10 +188,36 @@ __device__ __forceinline__ Split split_segment(uintptr_t p0, uintptr_t p1, uintp
 
 // dst = a + b over one tile of a segment.  Tile `tile` covers vectors
 // [tile*kThreads*U, (tile+1)*kThreads*U); tile 0 also does head and tail.
+// `aligned` (decided on the host for the whole launch): every operand starts on
+// a 16-byte boundary and n is a whole number of vectors, so there is no head,
+// no tail and nothing to decide per segment.
 template <class Op, int U, bool NTL, bool NTS>
 __device__ __forceinline__ void add_tile(void* dstp, const void* ap, const void* bp, size_t n,
-                                         size_t tile) {
+                                         size_t tile, bool aligned) {
   typedef typename Op::elem elem;
+  if (aligned) {
+    u32x4* dv = (u32x4*)dstp;
+    const u32x4* av = (const u32x4*)ap;
+    const u32x4* bv = (const u32x4*)bp;
+    const size_t nvec = n / Op::kPerVec;
+    const size_t v0 = tile * (size_t)(kThreads * U) + threadIdx.x;
+    if (v0 + (size_t)(U - 1) * kThreads < nvec) {
+      u32x4 x[U], y[U];
+#pragma unroll
+      for (int j = 0; j < U; ++j) x[j] = ld16<NTL>(av + v0 + (size_t)j * kThreads);
+#pragma unroll
+      for (int j = 0; j < U; ++j) y[j] = ld16<NTL>(bv + v0 + (size_t)j * kThreads);
+#pragma unroll
+      for (int j = 0; j < U; ++j) st16<NTS>(dv + v0 + (size_t)j * kThreads, Op::add(x[j], y[j]));
+    } else {
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const size_t v = v0 + (size_t)j * kThreads;
+        if (v < nvec) st16<NTS>(dv + v, Op::add(ld16<NTL>(av + v), ld16<NTL>(bv + v)));
+      }
+    }
+    return;
+  }
   const Split sp = split_segment((uintptr_t)dstp, (uintptr_t)ap, (uintptr_t)bp, n, sizeof(elem));
   elem* de = (elem*)dstp;
   const elem* ae = (const elem*)ap;
@@ -240,7 +266,28 @@ __device__ __forceinline__ void add_tile(void* dstp, const void* ap, const void*
 
 // Byte copy of one tile of a segment (same splitting, element = byte).
 template <int U, bool NTL, bool NTS>
-__device__ __forceinline__ void copy_tile(void* dstp, const void* srcp, size_t nbytes, size_t tile) {
+__device__ __forceinline__ void copy_tile(void* dstp, const void* srcp, size_t nbytes, size_t tile,
+                                          bool aligned = false) {
+  if (aligned) {   // 16-byte aligned ends on both sides: vectors only
+    u32x4* dv = (u32x4*)dstp;
+    const u32x4* sv = (const u32x4*)srcp;
+    const size_t nvec = nbytes / 16;
+    const size_t v0 = tile * (size_t)(kThreads * U) + threadIdx.x;
+    if (v0 + (size_t)(U - 1) * kThreads < nvec) {
+      u32x4 x[U];
+#pragma unroll
+      for (int j = 0; j < U; ++j) x[j] = ld16<NTL>(sv + v0 + (size_t)j * kThreads);
+#pragma unroll
+      for (int j = 0; j < U; ++j) st16<NTS>(dv + v0 + (size_t)j * kThreads, x[j]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const size_t v = v0 + (size_t)j * kThreads;
+        if (v < nvec) st16<NTS>(dv + v, ld16<NTL>(sv + v));
+      }
+    }
+    return;
+  }
   const Split sp = split_segment((uintptr_t)dstp, (uintptr_t)srcp, (uintptr_t)srcp, nbytes, 1);
   uint8_t* d8 = (uint8_t*)dstp;
   const uint8_t* s8 = (const uint8_t*)srcp;
@@ -317,7 +364,7 @@ struct Pieces {
 // `count` segments: dst[s] = a[s] + b[s], piece by piece.
 template <class Op, int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_add_segs(AddSegs t, int count, Pieces pc,
-                                                       size_t tiles_per_piece) {
+                                                       size_t tiles_per_piece, int aligned) {
   typedef typename Op::elem elem;
   // work items are counted in 32 bits (the host refuses launches beyond 2^32 - 1)
   const uint32_t tpp = (uint32_t)tiles_per_piece;
@@ -332,7 +379,8 @@ __global__ __launch_bounds__(kThreads) void k_add_segs(AddSegs t, int count, Pie
     const size_t p1 = piece / pc.s2, p2 = piece - (uint32_t)p1 * pc.s2;
     add_tile<Op, U, NTL, NTS>((elem*)t.dst[s] + p1 * pc.d1 + p2 * pc.d2,
                               (const elem*)t.a[s] + p1 * pc.a1 + p2 * pc.a2,
-                              (const elem*)t.b[s] + p1 * pc.b1 + p2 * pc.b2, pc.len, tile);
+                              (const elem*)t.b[s] + p1 * pc.b1 + p2 * pc.b2, pc.len, tile,
+                              aligned != 0);
   }
 }
 
@@ -349,7 +397,7 @@ struct RhArgs {
 template <class Op, int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_rh_round(RhArgs t, int P, size_t B, int round,
                                                        int from_src, int to_outs,
-                                                       size_t tiles_per_seg) {
+                                                       size_t tiles_per_seg, int aligned) {
   typedef typename Op::elem elem;
   const int group = P >> round;
   const int half = group >> 1;
@@ -366,7 +414,7 @@ __global__ __launch_bounds__(kThreads) void k_rh_round(RhArgs t, int P, size_t B
     const elem* a = (const elem*)(from_src ? t.src[r] : t.bufs[r]) + off;
     const elem* b = (const elem*)(from_src ? t.src[partner] : t.bufs[partner]) + off;
     elem* d = to_outs ? (elem*)t.outs[r] : (elem*)t.bufs[r] + off;
-    add_tile<Op, U, NTL, NTS>(d, a, b, count, tile);
+    add_tile<Op, U, NTL, NTS>(d, a, b, count, tile, aligned != 0);
   }
 }
 
@@ -379,7 +427,7 @@ struct CopySegs {
 // `count` byte segments; tiles_per_seg is sized for the longest one.
 template <int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_copy_segs(CopySegs t, int count,
-                                                        size_t tiles_per_seg) {
+                                                        size_t tiles_per_seg, int aligned) {
   const uint32_t tps = (uint32_t)tiles_per_seg;
   const uint64_t total = (uint64_t)count * tps;
   const size_t tile_bytes = (size_t)kThreads * U * 16;
@@ -391,7 +439,7 @@ __global__ __launch_bounds__(kThreads) void k_copy_segs(CopySegs t, int count,
     // a tile past the end of a short segment has nothing to do (16 spare
     // bytes cover the head shift of the vector body)
     if (tile != 0 && tile * tile_bytes >= nb + 16) continue;
-    copy_tile<U, NTL, NTS>(t.dst[s], t.src[s], nb, tile);
+    copy_tile<U, NTL, NTS>(t.dst[s], t.src[s], nb, tile, aligned != 0);
   }
 }
 
@@ -403,7 +451,7 @@ struct CopyPairs {
 // `count` segments of s1*s2 pieces of pc.len BYTES each (strides in bytes).
 template <int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_copy_pieces(CopyPairs t, int count, Pieces pc,
-                                                          size_t tiles_per_piece) {
+                                                          size_t tiles_per_piece, int aligned) {
   // work items are counted in 32 bits (the host refuses launches beyond 2^32 - 1)
   const uint32_t tpp = (uint32_t)tiles_per_piece;
   const uint32_t per_seg = pc.s1 * pc.s2 * tpp;
@@ -416,7 +464,7 @@ __global__ __launch_bounds__(kThreads) void k_copy_pieces(CopyPairs t, int count
     const size_t tile = rem - piece * tpp;
     const size_t p1 = piece / pc.s2, p2 = piece - (uint32_t)p1 * pc.s2;
     copy_tile<U, NTL, NTS>((uint8_t*)t.dst[s] + p1 * pc.d1 + p2 * pc.d2,
-                           (const uint8_t*)t.src[s] + p1 * pc.a1 + p2 * pc.a2, pc.len, tile);
+                           (const uint8_t*)t.src[s] + p1 * pc.a1 + p2 * pc.a2, pc.len, tile, aligned != 0);
   }
 }
 
@@ -475,7 +523,7 @@ __global__ __launch_bounds__(kThreads) void k_gather_multicast(GatherArgs t, int
 template <int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_block_transpose(uint8_t* dst, const uint8_t* src,
                                                               size_t rows, size_t cols, size_t m,
-                                                              size_t tiles_per_seg) {
+                                                              size_t tiles_per_seg, int aligned) {
   const uint32_t tps = (uint32_t)tiles_per_seg;
   const uint64_t total = (uint64_t)rows * cols * tps;
   for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
@@ -484,7 +532,7 @@ __global__ __launch_bounds__(kThreads) void k_block_transpose(uint8_t* dst, cons
     const size_t tile = w - blk32 * tps;
     const size_t blk = blk32;
     const size_t c = blk32 / (uint32_t)rows, r = blk - c * rows;
-    copy_tile<U, NTL, NTS>(dst + blk * m, src + (r * cols + c) * m, m, tile);
+    copy_tile<U, NTL, NTS>(dst + blk * m, src + (r * cols + c) * m, m, tile, aligned != 0);
   }
 }
 

@@ -266,9 +266,10 @@ def test_every_launch_tuning_gives_the_same_bits(target, unroll, nt, grid_cap):
     import torch
     from pccl import kernels
     lib = target.native
-    saved = {k: lib.get_tuning(k) for k in ("unroll", "nt_load", "nt_store", "grid_cap")}
+    saved = {k: lib.get_tuning(k) for k in ("unroll", "unroll_copy", "nt_load", "nt_store", "grid_cap")}
     try:
         lib.set_tuning("unroll", unroll)
+        lib.set_tuning("unroll_copy", unroll)
         lib.set_tuning("nt_load", nt)
         lib.set_tuning("nt_store", nt)
         lib.set_tuning("grid_cap", grid_cap)
