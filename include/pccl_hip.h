@@ -262,7 +262,9 @@ int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream);
  * key: "grid_cap" (max workgroups per launch, 0 = one tile per workgroup),
  *      "unroll"   (128-bit vectors per thread per operand of the add kernels:
  *                  1, 2, 4 or 8), "unroll_copy" (the same for the copy kernels),
- *      "nt_load" / "nt_store" (0/1: non-temporal global loads / stores).
+ *      "nt_load" / "nt_store" (0/1: non-temporal global loads / stores),
+ *      "lds_pad" / "lds_pad_copy" / "lds_pad_kway" (bytes of unused LDS per
+ *                  workgroup, 0..65536: bounds the workgroups resident per CU).
  * Returns 0, or PCCL_HIP_EINVAL for an unknown key or value.  Process-wide. */
 int pccl_hip_set_tuning(const char* key, long value);
 long pccl_hip_get_tuning(const char* key);

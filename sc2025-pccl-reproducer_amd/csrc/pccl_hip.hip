@@ -47,7 +47,13 @@ int launch_status(const char* what) {
 
 std::atomic<long> g_grid_cap{0};
 std::atomic<long> g_unroll{4};        // vectors per thread and operand, add kernels
-std::atomic<long> g_unroll_copy{2};   // ... copy kernels (8 KiB per workgroup: best across 64 MiB - 2 GiB)
+std::atomic<long> g_unroll_copy{1};   // ... copy kernels (4 KiB per workgroup: best for the all_gather steps)
+// Unused dynamic LDS requested per workgroup, only to bound how many workgroups
+// share a CU (160 KiB of LDS): the fewer are resident, the narrower the address
+// window the chip streams from at any moment.  0 = as many as fit (8).
+std::atomic<long> g_lds_pad{0};        // add kernels
+std::atomic<long> g_lds_pad_copy{0};   // copy kernels
+std::atomic<long> g_lds_pad_kway{0};   // fused reduce
 std::atomic<long> g_nt_load{1};
 std::atomic<long> g_nt_store{1};
 
@@ -148,9 +154,9 @@ struct AddLaunch {
   void operator()() const {
     unsigned grid = grid_for((size_t)count * pc.s1 * pc.s2 * tiles);
     if (dtype == PCCL_HIP_F32)
-      hipLaunchKernelGGL((k_add_segs<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, pc, tiles, aligned);
+      hipLaunchKernelGGL((k_add_segs<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), (unsigned)g_lds_pad.load(), stream, *segs, count, pc, tiles, aligned);
     else
-      hipLaunchKernelGGL((k_add_segs<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, pc, tiles, aligned);
+      hipLaunchKernelGGL((k_add_segs<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), (unsigned)g_lds_pad.load(), stream, *segs, count, pc, tiles, aligned);
   }
 };
 
@@ -189,7 +195,7 @@ struct CopyLaunch {
   template <int U, bool NTL, bool NTS>
   void operator()() const {
     unsigned grid = grid_for((size_t)count * tiles);
-    hipLaunchKernelGGL((k_copy_segs<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, tiles, aligned);
+    hipLaunchKernelGGL((k_copy_segs<U, NTL, NTS>), dim3(grid), dim3(kThreads), (unsigned)g_lds_pad_copy.load(), stream, *segs, count, tiles, aligned);
   }
 };
 
@@ -217,7 +223,7 @@ struct CopyPiecesLaunch {
   template <int U, bool NTL, bool NTS>
   void operator()() const {
     unsigned grid = grid_for((size_t)count * pc.s1 * pc.s2 * tiles);
-    hipLaunchKernelGGL((k_copy_pieces<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *segs, count, pc, tiles, aligned);
+    hipLaunchKernelGGL((k_copy_pieces<U, NTL, NTS>), dim3(grid), dim3(kThreads), (unsigned)g_lds_pad_copy.load(), stream, *segs, count, pc, tiles, aligned);
   }
 };
 
@@ -245,10 +251,10 @@ struct RhLaunch {
   void operator()() const {
     unsigned grid = grid_for((size_t)P * tiles);
     if (dtype == PCCL_HIP_F32)
-      hipLaunchKernelGGL((k_rh_round<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *args, P, B, round, from_src,
+      hipLaunchKernelGGL((k_rh_round<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), (unsigned)g_lds_pad.load(), stream, *args, P, B, round, from_src,
                                                                     to_outs, tiles, aligned);
     else
-      hipLaunchKernelGGL((k_rh_round<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *args, P, B, round, from_src,
+      hipLaunchKernelGGL((k_rh_round<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), (unsigned)g_lds_pad.load(), stream, *args, P, B, round, from_src,
                                                                      to_outs, tiles, aligned);
   }
 };
@@ -295,7 +301,7 @@ struct KwayLaunch {
     static_assert(U == 1, "the fused reduce is launched with one vector per thread");
     unsigned grid = grid_for((size_t)nout * tiles);
 #define PCCL_KWAY(KV) \
-  hipLaunchKernelGGL((k_reduce_kway<Acc, KV, U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, *args, k, g, nout, n, first0, tiles)
+  hipLaunchKernelGGL((k_reduce_kway<Acc, KV, U, NTL, NTS>), dim3(grid), dim3(kThreads), (unsigned)g_lds_pad_kway.load(), stream, *args, k, g, nout, n, first0, tiles)
     if (order == PCCL_HIP_ORDER_RING) { PCCL_KWAY(0); return; }
     switch (k) {
       case 2: PCCL_KWAY(2); break;
@@ -368,6 +374,9 @@ int pccl_hip_set_tuning(const char* key, long value) {
     if (value != 1 && value != 2 && value != 4 && value != 8)
       return fail(PCCL_HIP_EINVAL, "set_tuning: unroll_copy must be 1, 2, 4 or 8");
     g_unroll_copy = value;
+  } else if (!strcmp(key, "lds_pad") || !strcmp(key, "lds_pad_copy") || !strcmp(key, "lds_pad_kway")) {
+    if (value < 0 || value > 65536) return fail(PCCL_HIP_EINVAL, "set_tuning: %s must be in [0, 65536]", key);
+    (!strcmp(key, "lds_pad") ? g_lds_pad : !strcmp(key, "lds_pad_copy") ? g_lds_pad_copy : g_lds_pad_kway) = value;
   } else if (!strcmp(key, "nt_load")) {
     g_nt_load = value != 0;
   } else if (!strcmp(key, "nt_store")) {
@@ -383,6 +392,9 @@ long pccl_hip_get_tuning(const char* key) {
   if (!strcmp(key, "grid_cap")) return g_grid_cap;
   if (!strcmp(key, "unroll")) return g_unroll;
   if (!strcmp(key, "unroll_copy")) return g_unroll_copy;
+  if (!strcmp(key, "lds_pad")) return g_lds_pad;
+  if (!strcmp(key, "lds_pad_copy")) return g_lds_pad_copy;
+  if (!strcmp(key, "lds_pad_kway")) return g_lds_pad_kway;
   if (!strcmp(key, "nt_load")) return g_nt_load;
   if (!strcmp(key, "nt_store")) return g_nt_store;
   return -1;
