@@ -478,7 +478,20 @@ def cpu_baseline(info):
             line = [l for l in p.stdout.splitlines() if l.startswith("{")]
             if p.returncode == 0 and line:
                 r = json.loads(line[-1])
+                vendor = None
+                if dtype == "f32" and cmd[0] == launcher:
+                    # the vendor collective the reference reaches with --library mpi
+                    # --pccl-disable-cpp-backend (pccl/reduce_scatter.py:197), same shape
+                    vcmd = [a if a != "ring" else "mpi_block" for a in cmd]
+                    try:
+                        pv = subprocess.run(vcmd, capture_output=True, text=True, timeout=400)
+                        vl = [l for l in pv.stdout.splitlines() if l.startswith("{")]
+                        if pv.returncode == 0 and vl:
+                            vendor = round(json.loads(vl[-1])["GBps"], 3)
+                    except Exception:                         # noqa: BLE001
+                        vendor = None
                 return {"value": round(r["GBps"], 3), "unit": "GB/s", "cores": ranks, "kind": "port",
+                        "mpi_reduce_scatter_block_GBps": vendor,
                         "ms_per_call": round(r["ms_per_call"], 3), "host_cores": host_cores,
                         "sample": f"{sample}: ring reduce_scatter of the reference "
                                   f"(pccl/src/reduce_scatter.cpp:101-155) on host buffers, {ranks} ranks = {ranks} "

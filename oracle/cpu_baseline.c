@@ -8,6 +8,11 @@
  * the work buffer, then per step exchange one region with a neighbour
  * (MPI_Sendrecv) and add it with the scalar loop of pccl/src/common.cu:5-10.
  *
+ * With -DUSE_MPI, "--alg mpi_block" times the vendor collective instead:
+ * MPI_Reduce_scatter_block on float, what the reference reaches with
+ * `--library mpi --pccl-disable-cpp-backend` (pccl/reduce_scatter.py:197).  Its
+ * summation order belongs to the MPI library, so it is timed, not compared.
+ *
  * Two transports, chosen at compile time:
  *   -DUSE_MPI : MPI_Sendrecv between MPI ranks (mpiexec -np P ...), the
  *               transport the reference uses;
@@ -188,15 +193,17 @@ static int run_rank(comm_t* c, const opts_t* o) {
   char* w2 = (char*)malloc(total * s + 64);
   if (!in || !out || !w1 || !w2) { fprintf(stderr, "rank %d: out of memory\n", c->rank); return 2; }
   fill_input(in, total, o->dtype, o->seed, c->rank, o->scale);
-  const int ring = strcmp(o->alg, "ring") == 0;
-  for (int i = 0; i < o->warmup; ++i) {
-    if (ring) ring_rs(c, out, in, o->B, o->dtype, w1, w2); else rh_rs(c, out, in, o->B, o->dtype, w1, w2);
-  }
-  comm_barrier(c);
   double t0 = now_s();
-  for (int i = 0; i < o->iters; ++i) {
+  const int ring = strcmp(o->alg, "ring") == 0;
+  const int vendor = strcmp(o->alg, "mpi_block") == 0;
+  for (int i = 0; i < o->warmup + o->iters; ++i) {
+    if (i == o->warmup) { comm_barrier(c); t0 = now_s(); }
+#ifdef USE_MPI
+    if (vendor) { MPI_Reduce_scatter_block(in, out, (int)o->B, MPI_FLOAT, MPI_SUM, MPI_COMM_WORLD); continue; }
+#endif
     if (ring) ring_rs(c, out, in, o->B, o->dtype, w1, w2); else rh_rs(c, out, in, o->B, o->dtype, w1, w2);
   }
+  (void)vendor;
   double dt = now_s() - t0;
   double worst = comm_max(c, dt);
   if (o->dump) {
@@ -245,8 +252,15 @@ int main(int argc, char** argv) {
     else if (!strcmp(a, "--dump")) { o.dump = v; ++i; }
     else { fprintf(stderr, "unknown argument %s\n", a); return 64; }
   }
-  if (strcmp(o.alg, "ring") && strcmp(o.alg, "recursive")) {
-    fprintf(stderr, "--alg must be ring or recursive\n");
+  if (strcmp(o.alg, "ring") && strcmp(o.alg, "recursive") && strcmp(o.alg, "mpi_block")) {
+    fprintf(stderr, "--alg must be ring, recursive or mpi_block\n");
+    return 64;
+  }
+#ifndef USE_MPI
+  if (!strcmp(o.alg, "mpi_block")) { fprintf(stderr, "--alg mpi_block needs the MPI build\n"); return 64; }
+#endif
+  if (!strcmp(o.alg, "mpi_block") && o.dtype != ORACLE_F32) {
+    fprintf(stderr, "--alg mpi_block is float only (MPI has no bfloat16)\n");
     return 64;
   }
 #ifdef USE_MPI
