@@ -456,10 +456,13 @@ def cpu_baseline(info):
     if ranks & (ranks - 1):
         ranks = 1 << (ranks.bit_length() - 1)
     if info["kernel"] == "k_add_segs" and ranks == info["P"]:
-        block, iters, sample = info["B"], 12, "the workload itself (same P, dtype and block size)"
+        block, sample = info["B"], "the workload itself (same P, dtype and block size)"
     else:
-        block, iters = (1 << 22) if dtype == "bf16" else (1 << 21), 60      # 8 MiB blocks
+        block = (1 << 22) if dtype == "bf16" else (1 << 21)                 # 8 MiB blocks
         sample = "a ring reduce_scatter of the same dtype with 8 MiB blocks"
+    # about ten seconds of timed calls, assuming ~15 GB/s of algorithmic bytes on the host
+    job_bytes = 3 * (ranks - 1) * block * (2 if dtype == "bf16" else 4) * ranks
+    iters = max(5, min(500, int(10.0 / max(job_bytes / 15e9, 1e-3))))
     args = ["--alg", "ring", "--dtype", dtype, "--block", str(block), "--warmup", "1", "--iters", str(iters),
             "--scale", "0.01" if dtype == "bf16" else "1.0"]
     launcher = None
