@@ -45,8 +45,15 @@ extern "C" {
 
 #define PCCL_HIP_ABI_VERSION 1
 
-/* Largest number of ranks / shards / segments one call accepts. */
+/* Largest number of segments / shards one LAUNCH takes (their pointers travel
+ * in the kernel arguments): the limit of the batched kernels, of every fused
+ * mode and of the 2-D entry points. */
 #define PCCL_HIP_MAX_RANKS 64
+
+/* Largest number of virtual ranks of the per-step (and faithful) modes of
+ * pccl_hip_reduce_scatter_virtual / pccl_hip_all_gather_virtual: a step over
+ * more than PCCL_HIP_MAX_RANKS ranks goes out as several launches. */
+#define PCCL_HIP_MAX_VIRTUAL_RANKS 4096
 
 /* Element types.  bf16 sums are computed as RNE_bf16(float(a) + float(b)) at
  * every hop, which is what torch.add does on bfloat16 tensors in the
@@ -183,7 +190,8 @@ int pccl_hip_block_transpose(void* dst, const void* src, size_t rows,
  *   algorithm  : "ring" or "recursive" (recursive needs P a power of two);
  *                any other string is an error, as at pccl.cpp:83.
  * The summation order of each output block is that of the named algorithm in
- * every mode.  1 <= P <= PCCL_HIP_MAX_RANKS. */
+ * every mode.  1 <= P <= PCCL_HIP_MAX_VIRTUAL_RANKS (PCCL_HIP_MAX_RANKS for
+ * PCCL_HIP_MODE_FUSED). */
 int pccl_hip_reduce_scatter_virtual(void* const* outputs,
                                     const void* const* inputs,
                                     void* const* work, int P, size_t B,
@@ -200,7 +208,8 @@ int pccl_hip_reduce_scatter_virtual(void* const* outputs,
  *                (the ring schedule the reference leaves to MPI_Allgather,
  *                pccl/all_gather.py:124-128).
  * PCCL_HIP_MODE_STEPS replays one batched copy per step;
- * PCCL_HIP_MODE_FUSED places every shard directly; FAITHFUL == STEPS. */
+ * PCCL_HIP_MODE_FUSED places every shard directly; FAITHFUL == STEPS.
+ * P limits as for pccl_hip_reduce_scatter_virtual. */
 int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs,
                                 int P, size_t block_bytes,
                                 const char* algorithm, int mode, void* stream);

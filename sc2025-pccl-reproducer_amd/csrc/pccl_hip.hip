@@ -20,6 +20,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <vector>
 
 #include "pccl_hip.h"
 
@@ -70,6 +71,7 @@ using namespace pccl_kernels;
 // ---------------------------------------------------------------------------
 // Kernels count their work items (tiles) in 32 bits.
 constexpr size_t kMaxWorkItems = 0xffffffffull;
+constexpr int kMaxVirtualRanks = PCCL_HIP_MAX_VIRTUAL_RANKS;
 
 int check_work_items(size_t segments, size_t tiles, const char* what) {
   if (tiles != 0 && segments > kMaxWorkItems / tiles)
@@ -333,6 +335,34 @@ int launch_kway(const KwayArgs& args, int k, int g, int nout, size_t n, int dtyp
   return launch_status(what);
 }
 
+// A step over more segments than one launch's kernel arguments hold goes out
+// as several launches; the segments of a step are hazard-free, so their order
+// does not matter.
+struct AddTriple { void* dst; const void* a; const void* b; };
+
+int launch_add_list(const std::vector<AddTriple>& list, size_t n, int dtype, hipStream_t stream,
+                    const char* what) {
+  for (size_t i0 = 0; i0 < list.size(); i0 += kMaxSeg) {
+    const int cnt = (int)(list.size() - i0 < (size_t)kMaxSeg ? list.size() - i0 : (size_t)kMaxSeg);
+    AddSegs segs;
+    for (int s = 0; s < cnt; ++s) { segs.dst[s] = list[i0 + s].dst; segs.a[s] = list[i0 + s].a; segs.b[s] = list[i0 + s].b; }
+    if (int rc = launch_add(segs, cnt, n, dtype, stream, what)) return rc;
+  }
+  return PCCL_HIP_OK;
+}
+
+struct CopyItem { void* dst; const void* src; size_t nbytes; };
+
+int launch_copy_list(const std::vector<CopyItem>& list, hipStream_t stream, const char* what) {
+  for (size_t i0 = 0; i0 < list.size(); i0 += kMaxSeg) {
+    const int cnt = (int)(list.size() - i0 < (size_t)kMaxSeg ? list.size() - i0 : (size_t)kMaxSeg);
+    CopySegs segs;
+    for (int s = 0; s < cnt; ++s) { segs.dst[s] = list[i0 + s].dst; segs.src[s] = list[i0 + s].src; segs.nbytes[s] = list[i0 + s].nbytes; }
+    if (int rc = launch_copy(segs, cnt, stream, what)) return rc;
+  }
+  return PCCL_HIP_OK;
+}
+
 bool pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 
 int check_table(const void* const* tab, int count, const char* what, const char* name) {
@@ -572,11 +602,15 @@ int pccl_hip_reduce_scatter_virtual(void* const* outputs, const void* const* inp
   const bool rec = !strcmp(algorithm, "recursive");
   if (!ring && !rec)
     return fail(PCCL_HIP_EINVAL, "Unknown algorithm specified for reduce_scatter_mpi: %s", algorithm);
-  if (P < 1 || P > kMaxSeg) return fail(PCCL_HIP_EINVAL, "%s: P = %d outside [1, %d]", what, P, kMaxSeg);
+  if (P < 1 || P > kMaxVirtualRanks)
+    return fail(PCCL_HIP_EINVAL, "%s: P = %d outside [1, %d]", what, P, kMaxVirtualRanks);
   if (rec && !pow2(P))
     return fail(PCCL_HIP_EINVAL, "%s: recursive halving needs a power-of-two P, got %d", what, P);
   if (mode != PCCL_HIP_MODE_STEPS && mode != PCCL_HIP_MODE_FUSED && mode != PCCL_HIP_MODE_FAITHFUL)
     return fail(PCCL_HIP_EINVAL, "%s: unknown mode %d", what, mode);
+  if (mode == PCCL_HIP_MODE_FUSED && P > kMaxSeg)
+    return fail(PCCL_HIP_EINVAL, "%s: the fused mode folds at most %d ranks in one launch, got P = %d", what,
+                kMaxSeg, P);
   if (int rc = check_table((const void* const*)outputs, P, what, "outputs")) return rc;
   if (int rc = check_table(inputs, P, what, "inputs")) return rc;
   const bool need_work = (mode == PCCL_HIP_MODE_FAITHFUL && P > 1) || (mode == PCCL_HIP_MODE_STEPS && P > 2);
@@ -600,42 +634,40 @@ int pccl_hip_reduce_scatter_virtual(void* const* outputs, const void* const* inp
   }
 
   const bool faithful = mode == PCCL_HIP_MODE_FAITHFUL;
+  std::vector<CopyItem> copies((size_t)P);
   if (faithful) {  // buf <- input
-    CopySegs c;
-    for (int r = 0; r < P; ++r) { c.dst[r] = work[r]; c.src[r] = inputs[r]; c.nbytes[r] = (size_t)P * B * es; }
-    if (int rc = launch_copy(c, P, st, what)) return rc;
+    for (int r = 0; r < P; ++r) copies[r] = CopyItem{work[r], inputs[r], (size_t)P * B * es};
+    if (int rc = launch_copy_list(copies, st, what)) return rc;
   }
+  auto copy_out = [&]() {   // output <- buf[rank]
+    for (int r = 0; r < P; ++r)
+      copies[r] = CopyItem{outputs[r], (const uint8_t*)work[r] + (size_t)r * B * es, B * es};
+    return launch_copy_list(copies, st, what);
+  };
+  std::vector<AddTriple> adds((size_t)P);
 
   if (ring) {
     for (int step = 0; step < P - 1; ++step) {
-      AddSegs segs;
       const bool first = step == 0, last = step == P - 2;
       for (int r = 0; r < P; ++r) {
         const int recv_idx = ((r - step - 2) % P + P) % P;
         const int source = (r - 1 + P) % P;
         const size_t off = (size_t)recv_idx * B * es;
         if (faithful) {
-          segs.dst[r] = (uint8_t*)work[r] + off;
-          segs.a[r] = segs.dst[r];
-          segs.b[r] = (const uint8_t*)work[source] + off;
+          adds[r].dst = (uint8_t*)work[r] + off;
+          adds[r].a = adds[r].dst;
+          adds[r].b = (const uint8_t*)work[source] + off;
         } else {
           // rank r's block recv_idx is still its input; the running sum of the
           // left neighbour is its input at step 0 and its work buffer after
-          segs.a[r] = (const uint8_t*)inputs[r] + off;
-          segs.b[r] = first ? (const uint8_t*)inputs[source] + off : (const uint8_t*)work[source] + off;
-          segs.dst[r] = last ? outputs[r] : (void*)((uint8_t*)work[r] + off);
+          adds[r].a = (const uint8_t*)inputs[r] + off;
+          adds[r].b = first ? (const uint8_t*)inputs[source] + off : (const uint8_t*)work[source] + off;
+          adds[r].dst = last ? outputs[r] : (void*)((uint8_t*)work[r] + off);
         }
       }
-      if (int rc = launch_add(segs, P, B, dtype, st, what)) return rc;
+      if (int rc = launch_add_list(adds, B, dtype, st, what)) return rc;
     }
-    if (faithful) {
-      CopySegs c;
-      for (int r = 0; r < P; ++r) {
-        c.dst[r] = outputs[r]; c.src[r] = (const uint8_t*)work[r] + (size_t)r * B * es; c.nbytes[r] = B * es;
-      }
-      return launch_copy(c, P, st, what);
-    }
-    return PCCL_HIP_OK;
+    return faithful ? copy_out() : PCCL_HIP_OK;
   }
 
   // recursive halving
@@ -644,18 +676,25 @@ int pccl_hip_reduce_scatter_virtual(void* const* outputs, const void* const* inp
   for (int round = 0; round < rounds; ++round) {
     const bool from_inputs = !faithful && round == 0;
     const bool to_outputs = !faithful && round == rounds - 1;
-    if (int rc = pccl_hip_rh_round(work, from_inputs ? inputs : nullptr, to_outputs ? outputs : nullptr, P,
-                                   B, round, dtype, stream))
-      return rc;
-  }
-  if (faithful) {
-    CopySegs c;
-    for (int r = 0; r < P; ++r) {
-      c.dst[r] = outputs[r]; c.src[r] = (const uint8_t*)work[r] + (size_t)r * B * es; c.nbytes[r] = B * es;
+    if (P <= kMaxSeg) {   // the pairwise kernel finds partner and halves from (rank, round) itself
+      if (int rc = pccl_hip_rh_round(work, from_inputs ? inputs : nullptr, to_outputs ? outputs : nullptr, P,
+                                     B, round, dtype, stream))
+        return rc;
+      continue;
     }
-    return launch_copy(c, P, st, what);
+    const int group = P >> round, half = group / 2;
+    const size_t count = (size_t)half * B;
+    for (int r = 0; r < P; ++r) {
+      const bool lower = (r % group) < half;
+      const int partner = lower ? r + half : r - half;
+      const size_t off = ((size_t)(r / group) * group * B + (lower ? 0 : count)) * es;
+      adds[r].a = from_inputs ? (const uint8_t*)inputs[r] + off : (const uint8_t*)work[r] + off;
+      adds[r].b = from_inputs ? (const uint8_t*)inputs[partner] + off : (const uint8_t*)work[partner] + off;
+      adds[r].dst = to_outputs ? outputs[r] : (void*)((uint8_t*)work[r] + off);
+    }
+    if (int rc = launch_add_list(adds, count, dtype, st, what)) return rc;
   }
-  return PCCL_HIP_OK;
+  return faithful ? copy_out() : PCCL_HIP_OK;
 }
 
 int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs, int P,
@@ -666,11 +705,15 @@ int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs,
   const bool rec = !strcmp(algorithm, "recursive");
   if (!ring && !rec)
     return fail(PCCL_HIP_EINVAL, "Unknown algorithm specified for all_gather_mpi: %s", algorithm);
-  if (P < 1 || P > kMaxSeg) return fail(PCCL_HIP_EINVAL, "%s: P = %d outside [1, %d]", what, P, kMaxSeg);
+  if (P < 1 || P > kMaxVirtualRanks)
+    return fail(PCCL_HIP_EINVAL, "%s: P = %d outside [1, %d]", what, P, kMaxVirtualRanks);
   if (rec && !pow2(P))
     return fail(PCCL_HIP_EINVAL, "%s: recursive doubling needs a power-of-two P, got %d", what, P);
   if (mode != PCCL_HIP_MODE_STEPS && mode != PCCL_HIP_MODE_FUSED && mode != PCCL_HIP_MODE_FAITHFUL)
     return fail(PCCL_HIP_EINVAL, "%s: unknown mode %d", what, mode);
+  if (mode == PCCL_HIP_MODE_FUSED && P > kMaxSeg)
+    return fail(PCCL_HIP_EINVAL, "%s: the fused mode places at most %d shards in one launch, got P = %d", what,
+                kMaxSeg, P);
   if (int rc = check_table((const void* const*)outputs, P, what, "outputs")) return rc;
   if (int rc = check_table(inputs, P, what, "inputs")) return rc;
   if (block_bytes == 0) return PCCL_HIP_OK;
@@ -683,11 +726,10 @@ int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs,
   }
 
   // out[r][r] <- in[r]   (pccl/src/all_gather.cpp:31-35)
-  CopySegs c;
-  for (int r = 0; r < P; ++r) {
-    c.dst[r] = (uint8_t*)outputs[r] + (size_t)r * block_bytes; c.src[r] = inputs[r]; c.nbytes[r] = block_bytes;
-  }
-  if (int rc = launch_copy(c, P, st, what)) return rc;
+  std::vector<CopyItem> c((size_t)P);
+  for (int r = 0; r < P; ++r)
+    c[r] = CopyItem{(uint8_t*)outputs[r] + (size_t)r * block_bytes, inputs[r], block_bytes};
+  if (int rc = launch_copy_list(c, st, what)) return rc;
 
   if (rec) {
     for (int seg = 1; seg < P; seg *= 2) {
@@ -696,11 +738,10 @@ int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs,
         const int group_start = (r / (2 * seg)) * (2 * seg);
         const size_t recv_off = (size_t)(r < partner ? group_start + seg : group_start) * block_bytes;
         // the partner's send offset equals this rank's receive offset
-        c.dst[r] = (uint8_t*)outputs[r] + recv_off;
-        c.src[r] = (const uint8_t*)outputs[partner] + recv_off;
-        c.nbytes[r] = (size_t)seg * block_bytes;
+        c[r] = CopyItem{(uint8_t*)outputs[r] + recv_off, (const uint8_t*)outputs[partner] + recv_off,
+                        (size_t)seg * block_bytes};
       }
-      if (int rc = launch_copy(c, P, st, what)) return rc;
+      if (int rc = launch_copy_list(c, st, what)) return rc;
     }
     return PCCL_HIP_OK;
   }
@@ -709,11 +750,10 @@ int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs,
     for (int r = 0; r < P; ++r) {
       const int j = ((r - step - 1) % P + P) % P;
       const int source = (r - 1 + P) % P;
-      c.dst[r] = (uint8_t*)outputs[r] + (size_t)j * block_bytes;
-      c.src[r] = (const uint8_t*)outputs[source] + (size_t)j * block_bytes;
-      c.nbytes[r] = block_bytes;
+      c[r] = CopyItem{(uint8_t*)outputs[r] + (size_t)j * block_bytes,
+                      (const uint8_t*)outputs[source] + (size_t)j * block_bytes, block_bytes};
     }
-    if (int rc = launch_copy(c, P, st, what)) return rc;
+    if (int rc = launch_copy_list(c, st, what)) return rc;
   }
   return PCCL_HIP_OK;
 }

@@ -25,7 +25,8 @@ MODE_STEPS = 0
 MODE_FUSED = 1
 MODE_FAITHFUL = 2
 
-MAX_RANKS = 64
+MAX_RANKS = 64            # per launch / fused modes / 2-D grids
+MAX_VIRTUAL_RANKS = 4096  # per-step modes of the 1-D collectives
 ABI_VERSION = 1
 
 LIB_NAME = "libpccl_hip.so"

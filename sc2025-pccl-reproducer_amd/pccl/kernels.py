@@ -15,7 +15,7 @@ import torch
 
 from . import _native
 from ._native import (BF16, F32, MODE_FAITHFUL, MODE_FUSED, MODE_STEPS, ORDER_HALVING,
-                      ORDER_RING, MAX_RANKS)
+                      ORDER_RING, MAX_RANKS, MAX_VIRTUAL_RANKS)
 
 _MODES = {"steps": MODE_STEPS, "fused": MODE_FUSED, "faithful": MODE_FAITHFUL}
 
@@ -179,8 +179,9 @@ def reduce_scatter_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[torch
     P = len(inputs)
     if len(outputs) != P or P < 1:
         raise ValueError("need one output per input rank")
-    if P > MAX_RANKS:
-        raise RuntimeError(f"at most {MAX_RANKS} virtual ranks per communicator")
+    if P > (MAX_RANKS if mode_code(mode) == MODE_FUSED else MAX_VIRTUAL_RANKS):
+        raise RuntimeError(f"at most {MAX_VIRTUAL_RANKS} virtual ranks per communicator "
+                           f"({MAX_RANKS} in fused mode)")
     for t in inputs:
         check_device_tensor(t, "input")
     for t in outputs:
@@ -266,8 +267,9 @@ def all_gather_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[torch.Ten
     P = len(inputs)
     if len(outputs) != P or P < 1:
         raise ValueError("need one output per input rank")
-    if P > MAX_RANKS:
-        raise RuntimeError(f"at most {MAX_RANKS} virtual ranks per communicator")
+    if P > (MAX_RANKS if mode_code(mode) == MODE_FUSED else MAX_VIRTUAL_RANKS):
+        raise RuntimeError(f"at most {MAX_VIRTUAL_RANKS} virtual ranks per communicator "
+                           f"({MAX_RANKS} in fused mode)")
     for t in inputs:
         check_device_tensor(t, "input")
     for t in outputs:

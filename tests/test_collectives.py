@@ -42,6 +42,30 @@ def test_reduce_scatter_driver(target, dtype, mode, alg, P):
         assert_bits_equal(to_numpy(t_in[r], dtype), ins[r], f"input of rank {r} modified")
 
 
+@pytest.mark.parametrize("alg,P", [("ring", 65), ("ring", 100), ("recursive", 128)])
+@pytest.mark.parametrize("mode", ["steps", "faithful"])
+def test_more_ranks_than_one_launch_holds(target, alg, P, mode):
+    """Beyond 64 ranks a step goes out as several launches."""
+    import torch
+    from pccl import kernels
+    B, dtype = 21, O.BF16
+    ins = make_inputs(P, P * B, dtype, seed=77)
+    t_in = [to_torch(x, dtype, target.device) for x in ins]
+    t_out = [torch.zeros(B, dtype=torch.bfloat16, device=target.device) for _ in range(P)]
+    kernels.reduce_scatter_ranks(t_out, t_in, alg, mode)
+    target.sync()
+    want = _rs_oracle(alg)(ins, dtype)
+    for r in range(P):
+        assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"rank {r}")
+    g_out = [torch.zeros(P * B, dtype=torch.bfloat16, device=target.device) for _ in range(P)]
+    kernels.all_gather_ranks(g_out, t_out, alg, "steps")
+    target.sync()
+    for r in (0, P // 2, P - 1):
+        assert_bits_equal(to_numpy(g_out[r], dtype), np.concatenate(want), f"gather rank {r}")
+    with pytest.raises(RuntimeError, match="64 in fused mode"):
+        kernels.reduce_scatter_ranks(t_out, t_in, alg, "fused")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_config1_shape_small_ring_p4_uniform(target, dtype):
     """The P=4 fp32 workload at reduced length: uniform[-1,1], seed + rank;
