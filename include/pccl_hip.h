@@ -273,7 +273,8 @@ int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream);
  *                  1, 2, 4 or 8), "unroll_copy" (the same for the copy kernels),
  *      "nt_load" / "nt_store" (0/1: non-temporal global loads / stores),
  *      "lds_pad" / "lds_pad_copy" / "lds_pad_kway" (bytes of unused LDS per
- *                  workgroup, 0..65536: bounds the workgroups resident per CU).
+ *                  workgroup, 0..65536: bounds the workgroups resident per CU;
+ *                  lds_pad_kway = -1, the default, lets the fused reduce choose).
  * Returns 0, or PCCL_HIP_EINVAL for an unknown key or value.  Process-wide. */
 int pccl_hip_set_tuning(const char* key, long value);
 long pccl_hip_get_tuning(const char* key);
