@@ -239,6 +239,18 @@ class VirtualComm:
             kernels.reduce_scatter_ranks([p[1] for p in payloads], [p[0] for p in payloads], "ring", "fused")
         self._group.rendezvous.arrive(self._rank, "Reduce_scatter_block", (sendbuf, recvbuf), action)
 
+    def Bcast(self, buf: torch.Tensor, root: int = 0):
+        """MPI_Bcast (pccl/patch_deepspeed.py:80): the root's buffer is copied
+        into every other rank's buffer in one launch."""
+        def action(payloads):
+            src = payloads[root]
+            others = [p for i, p in enumerate(payloads) if i != root]
+            if others:
+                kernels.copy_batched([o.view(-1) for o in others], [src.view(-1)] * len(others))
+        if not 0 <= root < self._group.size:
+            raise VirtualRankError("Bcast: root outside the communicator")
+        self._group.rendezvous.arrive(self._rank, "Bcast", buf, action)
+
     def Free(self):
         pass
 

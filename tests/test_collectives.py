@@ -440,3 +440,78 @@ def test_request_wait_runs_epilogue(target):
     world.run(rank_main)
     assert sorted(called) == [0, 1]
     assert torch.equal(t_out[0], torch.cat(t_in))
+
+
+def test_patch_deepspeed_routes_world_collectives(target, monkeypatch):
+    """pccl/patch_deepspeed.py:95-126 against a stand-in for deepspeed's
+    TorchBackend (deepspeed itself is not installed): world-group SUM
+    collectives go through the 2-D PCCL path, the rest falls through."""
+    import enum
+    import sys
+    import types
+    import torch
+    import pccl
+    from pccl import build_kernels, patch_deepspeed as pd
+
+    class ReduceOp(enum.Enum):
+        SUM = 0
+        MAX = 1
+
+    fell_through = []
+
+    class TorchBackend:
+        def all_gather_into_tensor(self, o, i, group=None, async_op=False): fell_through.append("ag")
+        def reduce_scatter_tensor(self, o, i, op=None, group=None, async_op=False): fell_through.append("rs")
+        def all_reduce(self, t, op=None, group=None, async_op=False): fell_through.append("ar")
+        def broadcast(self, t, src, group=None, async_op=False): fell_through.append("bc")
+        def barrier(self, group=None, async_op=False, device_ids=None): fell_through.append("barrier")
+
+    ds = types.ModuleType("deepspeed"); comm_m = types.ModuleType("deepspeed.comm")
+    torch_m = types.ModuleType("deepspeed.comm.torch"); op_m = types.ModuleType("deepspeed.comm.reduce_op")
+    torch_m.TorchBackend = TorchBackend; op_m.ReduceOp = ReduceOp
+    for name, mod in (("deepspeed", ds), ("deepspeed.comm", comm_m), ("deepspeed.comm.torch", torch_m),
+                      ("deepspeed.comm.reduce_op", op_m)):
+        monkeypatch.setitem(sys.modules, name, mod)
+    monkeypatch.setattr(build_kernels, "build", lambda *a, **k: None)
+    monkeypatch.setattr(pd, "build", lambda *a, **k: None)
+
+    W, intra, m, dtype = 8, 4, 97, O.BF16
+    ins = make_inputs(W, W * m, dtype, seed=123)
+    t_in = [to_torch(x, dtype, target.device) for x in ins]
+    t_out = [torch.zeros(m, dtype=torch.bfloat16, device=target.device) for _ in range(W)]
+    g_out = [torch.zeros(W * m, dtype=torch.bfloat16, device=target.device) for _ in range(W)]
+    ar = [to_torch(x, dtype, target.device) for x in make_inputs(W, 64, dtype, seed=5)]
+    ar_in = make_inputs(W, 64, dtype, seed=5)
+    bc = [torch.full((33,), float(r), device=target.device) for r in range(W)]
+    world = pccl.VirtualWorld(W, target.device)
+
+    def rank_main(comm):
+        r = comm.Get_rank()
+        pd.patch_deepspeed(intra, comm=comm)
+        be = TorchBackend()
+        assert be.reduce_scatter_tensor(t_out[r], t_in[r], op=ReduceOp.SUM, async_op=True).wait() is None
+        be.all_gather_into_tensor(g_out[r], t_out[r])
+        be.all_reduce(ar[r], op=ReduceOp.SUM)
+        be.broadcast(bc[r], 3)
+        be.barrier()
+        if r == 0:      # not the world group / not a sum: the original methods run
+            be.reduce_scatter_tensor(t_out[r], t_in[r], op=ReduceOp.MAX)
+            be.all_gather_into_tensor(g_out[r], t_out[r], group=comm.world.subcomm([0, 1], 0))
+
+    world.run(rank_main)
+    target.sync()
+    assert fell_through == ["rs", "ag"]
+    want = O.reduce_scatter_2d(ins, intra, W // intra, dtype, "recursive")
+    want_ar = O.all_reduce(ar_in, dtype, "recursive")
+    for r in range(W):
+        assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"reduce_scatter rank {r}")
+        assert_bits_equal(to_numpy(g_out[r], dtype), np.concatenate(want), f"all_gather rank {r}")
+        assert_bits_equal(to_numpy(ar[r], dtype), want_ar[r], f"all_reduce rank {r}")
+        assert bool((bc[r] == 3.0).all())
+
+
+def test_patch_deepspeed_without_deepspeed_raises(target):
+    import pccl
+    from pccl import patch_deepspeed as pd
+    with pytest.raises(RuntimeError, match="needs the deepspeed package"):
+        pd.patch_deepspeed(2, comm=pccl.VirtualWorld(2, target.device).comm(0))
