@@ -330,12 +330,19 @@ struct KwayLaunch {
 int launch_kway(const KwayArgs& args, int k, int g, int nout, size_t n, int dtype, int order,
                 int first0, int per_hop, hipStream_t stream, const char* what) {
   if (n == 0 || nout == 0) return PCCL_HIP_OK;
-  // A one-level ring fold over 16 or more shards keeps nine loads per thread in
-  // flight; five resident workgroups per CU instead of eight (32 KiB of unused
-  // LDS each) narrow the streamed window and measured 3-7 % faster on MI355X for
-  // k = 16, 32, 64, while smaller k and the butterfly order lose from it.
+  // Fewer resident workgroups per CU (unused LDS takes the room) narrow the
+  // window each of the k streams has in flight.  Measured on MI355X, 4 GiB read:
+  // five per CU (32 KiB each) for one-level ring folds over 16 or more shards,
+  // +3-5 %; six per CU (24 KiB) for fp32 folds over 8-15 shards, +7 %; bf16
+  // below 16 shards, folds over fewer than 8 and the butterfly order lose from it.
   long pad = g_lds_pad_kway.load(std::memory_order_relaxed);
-  if (pad < 0) pad = (order == PCCL_HIP_ORDER_RING && g >= k && k >= 16) ? 32768 : 0;
+  if (pad < 0) {
+    pad = 0;
+    if (order == PCCL_HIP_ORDER_RING && g >= k) {
+      if (k >= 16) pad = 32768;
+      else if (k >= 8 && dtype == PCCL_HIP_F32) pad = 24576;
+    }
+  }
   KwayLaunch l{&args, k, g, nout, dtype, order, first0, per_hop, n, tiles_for(n * esize_of(dtype), 1),
                (unsigned)pad, stream};
   if (int rc = check_work_items((size_t)nout, l.tiles, what)) return rc;

@@ -591,23 +591,32 @@ __device__ __forceinline__ void tree_sum(Load& load, int first, float* out) {
   }
 }
 
-// Left fold over `count` operands in cyclic order first, first+1, ...; loads
-// are issued in batches of eight ahead of the adds.  load(q, f) fills the L
-// fp32 lanes of operand q; acc receives the result.
+// Left fold over `count` operands in cyclic order first, first+1, ...
+// load(q, f) fills the L fp32 lanes of operand q; acc receives the result.
+// Folds over kFoldPairedFrom or more operands issue their loads two at a time
+// ahead of the adds, shorter ones one at a time: with the workgroups a CU holds,
+// that keeps about as many bytes in flight as the memory system needs, and
+// deeper batches measured slower on MI355X (the streams of the k shards then
+// interleave more finely at the DRAM).
+constexpr int kFoldBatch = 2;
+constexpr int kFoldPairedFrom = 16;
+
 template <class Acc, int L, class Load>
 __device__ __forceinline__ void ring_fold(Load&& load, int count, int first, float* acc) {
   int q = first;
   load(q, acc);
   int done = 1;
-  for (; done + 8 <= count; done += 8) {
-    float f[8][L];
+  if (count >= kFoldPairedFrom) {
+    for (; done + kFoldBatch <= count; done += kFoldBatch) {
+      float f[kFoldBatch][L];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      q = q + 1 == count ? 0 : q + 1;
-      load(q, f[i]);
+      for (int i = 0; i < kFoldBatch; ++i) {
+        q = q + 1 == count ? 0 : q + 1;
+        load(q, f[i]);
+      }
+#pragma unroll
+      for (int i = 0; i < kFoldBatch; ++i) Acc::template hop_lanes<L>(acc, f[i]);
     }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) Acc::template hop_lanes<L>(acc, f[i]);
   }
   for (; done < count; ++done) {
     q = q + 1 == count ? 0 : q + 1;
