@@ -272,9 +272,15 @@ int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream);
  *      "unroll"   (128-bit vectors per thread per operand of the add kernels:
  *                  1, 2, 4 or 8), "unroll_copy" (the same for the copy kernels),
  *      "nt_load" / "nt_store" (0/1: non-temporal global loads / stores),
- *      "lds_pad" / "lds_pad_copy" / "lds_pad_kway" (bytes of unused LDS per
- *                  workgroup, 0..65536: bounds the workgroups resident per CU;
- *                  lds_pad_kway = -1, the default, lets the fused reduce choose).
+ *      "lds_pad" / "lds_pad_copy" / "lds_pad_kway" / "lds_pad_gather" (bytes of
+ *                  unused LDS per workgroup, 0..65536: bounds the workgroups
+ *                  resident per CU; lds_pad_kway = -1, the default, lets the
+ *                  fused reduce choose),
+ *      "unroll_gather" (vectors per thread of the multicast gather: 1, 2, 4, 8),
+ *      "gather_split"  (workgroups sharing one shard tile of the multicast
+ *                  gather, each storing to 1/gather_split of the outputs;
+ *                  0, the default = four outputs per workgroup),
+ *      "gather_nt" (0/1: non-temporal stores in the multicast gather).
  * Returns 0, or PCCL_HIP_EINVAL for an unknown key or value.  Process-wide. */
 int pccl_hip_set_tuning(const char* key, long value);
 long pccl_hip_get_tuning(const char* key);

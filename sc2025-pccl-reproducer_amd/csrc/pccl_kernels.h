@@ -476,17 +476,21 @@ struct GatherArgs {
 };
 
 // Direct all_gather placement for all P ranks: a workgroup reads one tile of
-// shard k ONCE and stores it into every rank's output at dst_off[k], so the
-// shards are fetched from HBM once instead of P times.
+// shard k and stores it into the outputs of one of `split` groups of ranks at
+// dst_off[k].  With split == 1 every shard byte is read once; with more groups
+// the same tile is read by `split` workgroups launched side by side, each with
+// nout / split write streams.
 template <int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_gather_multicast(GatherArgs t, int P, int nout,
-                                                              size_t tiles_per_seg) {
+                                                              size_t tiles_per_seg, int split) {
   const uint32_t tps = (uint32_t)tiles_per_seg;
-  const uint64_t total = (uint64_t)P * tps;
+  const uint64_t total = (uint64_t)P * tps * (uint32_t)split;
   const size_t tile_bytes = (size_t)kThreads * U * 16;
   const unsigned tid = threadIdx.x;
   for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
-    const uint32_t w = (uint32_t)w64;
+    const uint32_t w = (uint32_t)w64 / (uint32_t)split;
+    const int grp = (int)((uint32_t)w64 - w * (uint32_t)split);
+    const int r0 = (int)((long)nout * grp / split), r1 = (int)((long)nout * (grp + 1) / split);
     const int k = (int)(w / tps);
     const size_t tile = w - (uint32_t)k * tps;
     const size_t nb = t.nbytes[k];
@@ -495,7 +499,7 @@ __global__ __launch_bounds__(kThreads) void k_gather_multicast(GatherArgs t, int
     const size_t off = t.dst_off[k];
     // vector path only if the source and EVERY destination share alignment
     bool aligned = ((uintptr_t)src & 15u) == 0 && (off & 15u) == 0;
-    for (int r = 0; r < nout; ++r) aligned = aligned && (((uintptr_t)t.outs[r]) & 15u) == 0;
+    for (int r = r0; r < r1; ++r) aligned = aligned && (((uintptr_t)t.outs[r]) & 15u) == 0;
     const size_t nvec = nb / 16;
     const size_t base = tile * (size_t)(kThreads * U);
     if (aligned && base + (size_t)kThreads * U <= nvec) {
@@ -503,17 +507,17 @@ __global__ __launch_bounds__(kThreads) void k_gather_multicast(GatherArgs t, int
       u32x4 x[U];
 #pragma unroll
       for (int j = 0; j < U; ++j) x[j] = ld16<NTL>(sv + base + (size_t)j * kThreads + tid);
-      for (int r = 0; r < nout; ++r) {
+      for (int r = r0; r < r1; ++r) {
         u32x4* dv = (u32x4*)((uint8_t*)t.outs[r] + off);
 #pragma unroll
         for (int j = 0; j < U; ++j) st16<NTS>(dv + base + (size_t)j * kThreads + tid, x[j]);
       }
       if (tile == 0 && tid < nb - nvec * 16) {   // the last nb % 16 bytes of the shard
         const size_t i = nvec * 16 + tid;
-        for (int r = 0; r < nout; ++r) ((uint8_t*)t.outs[r])[off + i] = src[i];
+        for (int r = r0; r < r1; ++r) ((uint8_t*)t.outs[r])[off + i] = src[i];
       }
     } else {
-      for (int r = 0; r < nout; ++r)
+      for (int r = r0; r < r1; ++r)
         copy_tile<U, NTL, NTS>((uint8_t*)t.outs[r] + off, src, nb, tile);
     }
   }

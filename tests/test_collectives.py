@@ -171,6 +171,40 @@ def test_all_gather_uneven_padded_to_256(target):
     assert torch.equal(got, torch.cat([as_bytes(t) for t in t_in]))
 
 
+@pytest.mark.parametrize("P", [1, 3, 5, 16])
+@pytest.mark.parametrize("split", [0, 1, 2, 3, 64])
+@pytest.mark.parametrize("unroll,nt", [(1, 1), (4, 0)])
+def test_multicast_gather_tunings_give_the_same_bytes(target, P, split, unroll, nt):
+    """However the outputs of a shard tile are shared among workgroups
+    (gather_split), the gathered bytes are the same; ragged lengths and odd
+    rank counts included."""
+    import torch
+    from pccl import kernels
+    lib = target.native
+    keys = ("gather_split", "unroll_gather", "gather_nt")
+    saved = {k: lib.get_tuning(k) for k in keys}
+    rng = np.random.default_rng(100 + P)
+    nbytes = [int(x) for x in rng.integers(0, 30_000, P)]
+    nbytes[0] = 4096 * 3 + 5
+    t_in = [torch.from_numpy(rng.integers(0, 256, n, dtype=np.uint8)).to(target.device) for n in nbytes]
+    off = kernels.padded_offsets(nbytes, 16)
+    total = off[-1] + nbytes[-1] + 7
+    try:
+        lib.set_tuning("gather_split", split)
+        lib.set_tuning("unroll_gather", unroll)
+        lib.set_tuning("gather_nt", nt)
+        t_out = [torch.full((total,), 0x5A, dtype=torch.uint8, device=target.device) for _ in range(P)]
+        lib.all_gather_uneven_virtual([t.data_ptr() for t in t_out], [t.data_ptr() for t in t_in], nbytes, off,
+                                      target.stream())
+        target.sync()
+    finally:
+        for k, v in saved.items():
+            lib.set_tuning(k, v)
+    want = O.uneven_all_gather([t.cpu().numpy() for t in t_in], off, total, fill=0x5A)
+    for r in range(P):
+        assert np.array_equal(t_out[r].cpu().numpy(), want[r]), f"rank {r}"
+
+
 def _golden_cases():
     import glob
     import os
