@@ -574,6 +574,7 @@ def main():
     start = torch.cuda.Event(enable_timing=True)
     end = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    launches0 = lib.launch_count()
     start.record(stream)
     for _ in range(args.steps):
         step()
@@ -581,6 +582,8 @@ def main():
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     dev_ms = start.elapsed_time(end)
+    # a step of a schedule goes out as several launches of bounded size (launch_mib)
+    launched = (lib.launch_count() - launches0) / args.steps
     ms_per_step = dev_ms / args.steps
     value = info["alg_bytes"] / (ms_per_step * 1e-3) / 1e9
 
@@ -598,17 +601,18 @@ def main():
         ok = bool(info["verify"]())
 
     # the timed region holds nothing but the dominant kernel's launches (plus, in
-    # faithful mode, the copies), so its mean launch time is region / launches
-    if info["launches"] == info["kernel_launches"]:
-        kernel_ms = dev_ms / (args.steps * info["kernel_launches"])
-    elif info["kernel_bytes"] == info["alg_bytes"]:
-        # launches of different sizes (halving rounds): bytes and time of the whole sequence
-        kernel_ms = dev_ms / args.steps
+    # faithful mode, the copies), so its mean launch time is region / launches and
+    # the bytes of a mean launch are the step's kernel bytes / launches
+    if info["launches"] == info["kernel_launches"] or info["kernel_bytes"] == info["alg_bytes"]:
+        step_kernel_bytes = (info["kernel_bytes"] * info["kernel_launches"]
+                             if info["launches"] == info["kernel_launches"] else info["kernel_bytes"])
+        kernel_ms = dev_ms / (args.steps * launched)
+        launch_bytes = step_kernel_bytes / launched
     else:
         kernel_ms = None
     roof = None
     if kernel_ms:
-        achieved = info["kernel_bytes"] / (kernel_ms * 1e-3) / 1e9
+        achieved = launch_bytes / (kernel_ms * 1e-3) / 1e9
         traffic = None
         tfile = os.path.join(ROOT, "profiles", "traffic.json")
         if os.path.exists(tfile):
@@ -618,7 +622,7 @@ def main():
                 traffic = None
         roof = {"bound": "hbm", "kernel": info["kernel"], "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                "traffic": traffic, "bytes_per_launch": info["kernel_bytes"],
+                "traffic": traffic, "bytes_per_launch": int(round(launch_bytes)),
                 "avg_launch_ms": round(kernel_ms, 5)}
 
     cpu = None if args.no_cpu_baseline else cpu_baseline(info)
@@ -628,9 +632,9 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": info["dtype"], "data": "synthetic",
         "config": {"workload": f"{args.workload}: {info['desc']}", "algorithmic_bytes_per_step": info["alg_bytes"],
-                   "launches_per_step": info["launches"], "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
+                   "launches_per_step": launched, "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
                    "wall_ms_per_step": round(wall_ms / args.steps, 4), "verified": ok,
-                   "tuning": {k: lib.get_tuning(k) for k in ("grid_cap", "unroll", "unroll_copy", "nt_load", "nt_store")}},
+                   "tuning": {k: lib.get_tuning(k) for k in ("grid_cap", "unroll", "unroll_copy", "nt_load", "nt_store", "launch_mib")}},
         "roofline": roof, "cpu_baseline": cpu,
     }
     print(json.dumps(out), flush=True)

@@ -280,10 +280,20 @@ int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream);
  *      "gather_split"  (workgroups sharing one shard tile of the multicast
  *                  gather, each storing to 1/gather_split of the outputs;
  *                  0, the default = four outputs per workgroup),
- *      "gather_nt" (0/1: non-temporal stores in the multicast gather).
+ *      "gather_nt" (0/1: non-temporal stores in the multicast gather),
+ *      "launch_mib" (a step of the add kernels goes out as equal launches that
+ *                  move about this many MiB each, a fused reduce over at most
+ *                  16 shards as launches 1.5 times as large; 0 = always one
+ *                  launch; default 1024.  Copies are always one launch).
  * Returns 0, or PCCL_HIP_EINVAL for an unknown key or value.  Process-wide. */
 int pccl_hip_set_tuning(const char* key, long value);
 long pccl_hip_get_tuning(const char* key);
+
+/* Kernel launches this process has issued through the library so far (a step
+ * of a schedule may be several, see "launch_mib").  For measurement: the
+ * difference around a timed region is the number of launches in it.  No
+ * counterpart in the reference. */
+unsigned long long pccl_hip_launch_count(void);
 
 #ifdef __cplusplus
 }

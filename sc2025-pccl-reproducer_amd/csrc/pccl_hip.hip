@@ -59,6 +59,8 @@ std::atomic<long> g_lds_pad_gather{0}; // multicast gather
 std::atomic<long> g_gather_split{0};   // groups of outputs per shard tile in the multicast gather; 0 = four outputs a group
 std::atomic<long> g_gather_nt{1};      // non-temporal stores in the multicast gather
 std::atomic<long> g_unroll_gather{1};  // vectors per thread in the multicast gather
+std::atomic<unsigned long long> g_launches{0};   // kernel launches issued so far
+std::atomic<long> g_launch_mib{1024};  // traffic per launch of the add kernels, MiB (0 = a step is one launch whatever its size)
 std::atomic<long> g_nt_load{1};
 std::atomic<long> g_nt_store{1};
 
@@ -92,6 +94,35 @@ unsigned grid_for(size_t total_tiles) {
   if (g == 0) g = 1;
   return (unsigned)g;
 }
+
+// Calls launch(span, grid) for consecutive, equal spans of the `items` work
+// items of a schedule step, each moving about target_mib MiB (item_bytes per
+// work item; 0 = one span); span bounds are multiples of `multiple`.
+// On MI355X the add kernels slow down over the length of a launch: 12 GiB of
+// traffic in one launch runs at 6.0 TB/s, as launches of 0.75-1.5 GiB at 6.4;
+// pieces under 0.5 GiB lose again to the drain at the end of every launch.
+// Copies and the multicast gather do not show it; the fused reduce gains 2 %
+// for 8 and 16 shards and loses for 32 (its workgroups live k loads long, and
+// so does the drain), see launch_kway.
+template <class F>
+void for_spans(size_t items, size_t item_bytes, size_t multiple, long target_mib, F&& launch) {
+  if (items == 0) return;
+  size_t per = items;
+  if (target_mib > 0 && item_bytes > 0) {
+    const double total = (double)items * (double)item_bytes;
+    size_t pieces = (size_t)(total / ((double)target_mib * 1048576.0) + 0.5);
+    if (pieces < 1) pieces = 1;
+    per = (items + pieces - 1) / pieces;
+    per = (per + multiple - 1) / multiple * multiple;
+  }
+  for (size_t w0 = 0; w0 < items; w0 += per) {
+    const size_t w1 = items - w0 < per ? items : w0 + per;
+    launch(Span{(uint32_t)w0, (uint32_t)w1}, grid_for(w1 - w0));
+    g_launches.fetch_add(1, std::memory_order_relaxed);
+  }
+}
+
+long add_launch_mib() { return g_launch_mib.load(std::memory_order_relaxed); }
 
 size_t tiles_for(size_t nbytes, int unroll) {
   // one extra vector covers the shift of the body behind an unaligned head
@@ -158,11 +189,13 @@ struct AddLaunch {
   hipStream_t stream;
   template <int U, bool NTL, bool NTS>
   void operator()() const {
-    unsigned grid = grid_for((size_t)count * pc.s1 * pc.s2 * tiles);
-    if (dtype == PCCL_HIP_F32)
-      hipLaunchKernelGGL((k_add_segs<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), (unsigned)g_lds_pad.load(), stream, *segs, count, pc, tiles, aligned);
-    else
-      hipLaunchKernelGGL((k_add_segs<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), (unsigned)g_lds_pad.load(), stream, *segs, count, pc, tiles, aligned);
+    const unsigned lds = (unsigned)g_lds_pad.load();
+    for_spans((size_t)count * pc.s1 * pc.s2 * tiles, 3 * kTileBytes * U, 1, add_launch_mib(), [&](Span span, unsigned grid) {
+      if (dtype == PCCL_HIP_F32)
+        hipLaunchKernelGGL((k_add_segs<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *segs, count, pc, tiles, aligned, span);
+      else
+        hipLaunchKernelGGL((k_add_segs<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *segs, count, pc, tiles, aligned, span);
+    });
   }
 };
 
@@ -200,8 +233,10 @@ struct CopyLaunch {
   hipStream_t stream;
   template <int U, bool NTL, bool NTS>
   void operator()() const {
-    unsigned grid = grid_for((size_t)count * tiles);
-    hipLaunchKernelGGL((k_copy_segs<U, NTL, NTS>), dim3(grid), dim3(kThreads), (unsigned)g_lds_pad_copy.load(), stream, *segs, count, tiles, aligned);
+    const unsigned lds = (unsigned)g_lds_pad_copy.load();
+    for_spans((size_t)count * tiles, 2 * kTileBytes * U, 1, 0, [&](Span span, unsigned grid) {
+      hipLaunchKernelGGL((k_copy_segs<U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *segs, count, tiles, aligned, span);
+    });
   }
 };
 
@@ -228,8 +263,10 @@ struct CopyPiecesLaunch {
   hipStream_t stream;
   template <int U, bool NTL, bool NTS>
   void operator()() const {
-    unsigned grid = grid_for((size_t)count * pc.s1 * pc.s2 * tiles);
-    hipLaunchKernelGGL((k_copy_pieces<U, NTL, NTS>), dim3(grid), dim3(kThreads), (unsigned)g_lds_pad_copy.load(), stream, *segs, count, pc, tiles, aligned);
+    const unsigned lds = (unsigned)g_lds_pad_copy.load();
+    for_spans((size_t)count * pc.s1 * pc.s2 * tiles, 2 * kTileBytes * U, 1, 0, [&](Span span, unsigned grid) {
+      hipLaunchKernelGGL((k_copy_pieces<U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *segs, count, pc, tiles, aligned, span);
+    });
   }
 };
 
@@ -255,13 +292,13 @@ struct RhLaunch {
   hipStream_t stream;
   template <int U, bool NTL, bool NTS>
   void operator()() const {
-    unsigned grid = grid_for((size_t)P * tiles);
-    if (dtype == PCCL_HIP_F32)
-      hipLaunchKernelGGL((k_rh_round<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), (unsigned)g_lds_pad.load(), stream, *args, P, B, round, from_src,
-                                                                    to_outs, tiles, aligned);
-    else
-      hipLaunchKernelGGL((k_rh_round<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), (unsigned)g_lds_pad.load(), stream, *args, P, B, round, from_src,
-                                                                     to_outs, tiles, aligned);
+    const unsigned lds = (unsigned)g_lds_pad.load();
+    for_spans((size_t)P * tiles, 3 * kTileBytes * U, 1, add_launch_mib(), [&](Span span, unsigned grid) {
+      if (dtype == PCCL_HIP_F32)
+        hipLaunchKernelGGL((k_rh_round<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *args, P, B, round, from_src, to_outs, tiles, aligned, span);
+      else
+        hipLaunchKernelGGL((k_rh_round<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *args, P, B, round, from_src, to_outs, tiles, aligned, span);
+    });
   }
 };
 
@@ -275,11 +312,14 @@ struct GatherLaunch {
   // Plain loads whatever the tuning says; the stores follow their own setting.
   template <int U, bool NTL, bool NTS>
   void operator()() const {
-    unsigned grid = grid_for((size_t)P * tiles * (size_t)split);
-    if (nt)
-      hipLaunchKernelGGL((k_gather_multicast<U, false, true>), dim3(grid), dim3(kThreads), lds_pad, stream, *args, P, nout, tiles, split);
-    else
-      hipLaunchKernelGGL((k_gather_multicast<U, false, false>), dim3(grid), dim3(kThreads), lds_pad, stream, *args, P, nout, tiles, split);
+    // a work item reads a tile and stores it to its share of the outputs
+    const size_t item_bytes = kTileBytes * U * (1 + ((size_t)nout + split - 1) / split);
+    for_spans((size_t)P * tiles * (size_t)split, item_bytes, (size_t)split, 0, [&](Span span, unsigned grid) {
+      if (nt)
+        hipLaunchKernelGGL((k_gather_multicast<U, false, true>), dim3(grid), dim3(kThreads), lds_pad, stream, *args, P, nout, tiles, split, span);
+      else
+        hipLaunchKernelGGL((k_gather_multicast<U, false, false>), dim3(grid), dim3(kThreads), lds_pad, stream, *args, P, nout, tiles, split, span);
+    });
   }
 };
 
@@ -291,8 +331,9 @@ struct TransposeLaunch {
   hipStream_t stream;
   template <int U, bool NTL, bool NTS>
   void operator()() const {
-    unsigned grid = grid_for(rows * cols * tiles);
-    hipLaunchKernelGGL((k_block_transpose<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, dst, src, rows, cols, m, tiles, aligned);
+    for_spans(rows * cols * tiles, 2 * kTileBytes * U, 1, 0, [&](Span span, unsigned grid) {
+      hipLaunchKernelGGL((k_block_transpose<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, dst, src, rows, cols, m, tiles, aligned, span);
+    });
   }
 };
 
@@ -309,18 +350,19 @@ struct KwayLaunch {
   template <class Acc, int U, bool NTL, bool NTS>
   void run() const {
     static_assert(U == 1, "the fused reduce is launched with one vector per thread");
-    unsigned grid = grid_for((size_t)nout * tiles);
 #define PCCL_KWAY(KV) \
-  hipLaunchKernelGGL((k_reduce_kway<Acc, KV, U, NTL, NTS>), dim3(grid), dim3(kThreads), lds_pad, stream, *args, k, g, nout, n, first0, tiles)
-    if (order == PCCL_HIP_ORDER_RING) { PCCL_KWAY(0); return; }
-    switch (k) {
-      case 2: PCCL_KWAY(2); break;
-      case 4: PCCL_KWAY(4); break;
-      case 8: PCCL_KWAY(8); break;
-      case 16: PCCL_KWAY(16); break;
-      case 32: PCCL_KWAY(32); break;
-      default: PCCL_KWAY(64); break;
-    }
+  hipLaunchKernelGGL((k_reduce_kway<Acc, KV, U, NTL, NTS>), dim3(grid), dim3(kThreads), lds_pad, stream, *args, k, g, nout, n, first0, tiles, span)
+    for_spans((size_t)nout * tiles, kTileBytes * U * ((size_t)k + 1), 1, k <= 16 ? add_launch_mib() * 3 / 2 : 0, [&](Span span, unsigned grid) {
+      if (order == PCCL_HIP_ORDER_RING) { PCCL_KWAY(0); return; }
+      switch (k) {
+        case 2: PCCL_KWAY(2); break;
+        case 4: PCCL_KWAY(4); break;
+        case 8: PCCL_KWAY(8); break;
+        case 16: PCCL_KWAY(16); break;
+        case 32: PCCL_KWAY(32); break;
+        default: PCCL_KWAY(64); break;
+      }
+    });
 #undef PCCL_KWAY
   }
 
@@ -441,6 +483,9 @@ int pccl_hip_set_tuning(const char* key, long value) {
     if (value != 1 && value != 2 && value != 4 && value != 8)
       return fail(PCCL_HIP_EINVAL, "set_tuning: unroll_gather must be 1, 2, 4 or 8");
     g_unroll_gather = value;
+  } else if (!strcmp(key, "launch_mib")) {
+    if (value < 0) return fail(PCCL_HIP_EINVAL, "set_tuning: launch_mib must be >= 0");
+    g_launch_mib = value;
   } else if (!strcmp(key, "gather_nt")) {
     g_gather_nt = value != 0;
   } else if (!strcmp(key, "nt_load")) {
@@ -452,6 +497,8 @@ int pccl_hip_set_tuning(const char* key, long value) {
   }
   return PCCL_HIP_OK;
 }
+
+unsigned long long pccl_hip_launch_count(void) { return g_launches.load(std::memory_order_relaxed); }
 
 long pccl_hip_get_tuning(const char* key) {
   if (!key) return -1;
@@ -465,6 +512,7 @@ long pccl_hip_get_tuning(const char* key) {
   if (!strcmp(key, "gather_split")) return g_gather_split;
   if (!strcmp(key, "unroll_gather")) return g_unroll_gather;
   if (!strcmp(key, "gather_nt")) return g_gather_nt;
+  if (!strcmp(key, "launch_mib")) return g_launch_mib;
   if (!strcmp(key, "nt_load")) return g_nt_load;
   if (!strcmp(key, "nt_store")) return g_nt_store;
   return -1;
@@ -1081,15 +1129,22 @@ int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream) {
   if (nbytes < 4096) return fail(PCCL_HIP_EINVAL, "%s: buffer must hold at least 4096 bytes", what);
   if (!buf || ((uintptr_t)buf & 15u)) return fail(PCCL_HIP_EINVAL, "%s: buffer must be 16-byte aligned", what);
   const size_t nvec = nbytes / 16;
-  const size_t tiles = (nvec + (size_t)kThreads * 4 - 1) / ((size_t)kThreads * 4);
+  const size_t per_tile = (size_t)kThreads * 4;   // vectors per workgroup
+  const size_t tiles = (nvec + per_tile - 1) / per_tile;
   if (tiles > kMaxGrid) return fail(PCCL_HIP_EINVAL, "%s: buffer too large", what);
   hipStream_t st = (hipStream_t)stream;
-  if (kind == 0)
-    hipLaunchKernelGGL((k_probe_read<4, true>), dim3((unsigned)tiles), dim3(kThreads), 0, st,
-                       (const u32x4*)buf, (u32x4*)buf, nvec);
-  else
-    hipLaunchKernelGGL((k_probe_write<4, false>), dim3((unsigned)tiles), dim3(kThreads), 0, st, (u32x4*)buf,
-                       nvec, 0x3f803f80u);
+  for_spans(tiles, per_tile * 16, 1, 0, [&](Span span, unsigned) {
+    u32x4* p = (u32x4*)buf + (size_t)span.begin * per_tile;
+    const size_t left = nvec - (size_t)span.begin * per_tile;
+    const size_t cnt = (size_t)(span.end - span.begin) * per_tile;
+    const size_t nv = cnt < left ? cnt : left;
+    if (kind == 0)
+      hipLaunchKernelGGL((k_probe_read<4, true>), dim3(span.end - span.begin), dim3(kThreads), 0, st,
+                         (const u32x4*)p, (u32x4*)buf, nv);
+    else
+      hipLaunchKernelGGL((k_probe_write<4, false>), dim3(span.end - span.begin), dim3(kThreads), 0, st, p, nv,
+                         0x3f803f80u);
+  });
   return launch_status(what);
 }
 

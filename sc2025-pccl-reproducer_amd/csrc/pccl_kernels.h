@@ -13,7 +13,15 @@
 namespace pccl_kernels {
 
 constexpr int kThreads = 256;              // 4 waves of 64 lanes
+constexpr size_t kTileBytes = kThreads * 16;   // what a workgroup moves per operand with one vector per thread
 constexpr int kMaxSeg = PCCL_HIP_MAX_RANKS;
+
+// The work items [begin, end) one launch covers.  Long schedules go out as
+// several launches of bounded size: within one launch the XCDs drift apart in
+// the address range they stream from, and throughput falls with its length.
+struct Span {
+  uint32_t begin, end;
+};
 constexpr unsigned kMaxGrid = 0x7fffffffu;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -364,13 +372,12 @@ struct Pieces {
 // `count` segments: dst[s] = a[s] + b[s], piece by piece.
 template <class Op, int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_add_segs(AddSegs t, int count, Pieces pc,
-                                                       size_t tiles_per_piece, int aligned) {
+                                                       size_t tiles_per_piece, int aligned, Span span) {
   typedef typename Op::elem elem;
   // work items are counted in 32 bits (the host refuses launches beyond 2^32 - 1)
   const uint32_t tpp = (uint32_t)tiles_per_piece;
   const uint32_t per_seg = pc.s1 * pc.s2 * tpp;
-  const uint64_t total = (uint64_t)count * per_seg;
-  for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
+  for (uint64_t w64 = (uint64_t)span.begin + blockIdx.x; w64 < span.end; w64 += gridDim.x) {
     const uint32_t w = (uint32_t)w64;
     const uint32_t s = w / per_seg;
     const uint32_t rem = w - s * per_seg;
@@ -397,14 +404,13 @@ struct RhArgs {
 template <class Op, int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_rh_round(RhArgs t, int P, size_t B, int round,
                                                        int from_src, int to_outs,
-                                                       size_t tiles_per_seg, int aligned) {
+                                                       size_t tiles_per_seg, int aligned, Span span) {
   typedef typename Op::elem elem;
   const int group = P >> round;
   const int half = group >> 1;
   const size_t count = (size_t)half * B;
   const uint32_t tps = (uint32_t)tiles_per_seg;
-  const uint64_t total = (uint64_t)P * tps;
-  for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
+  for (uint64_t w64 = (uint64_t)span.begin + blockIdx.x; w64 < span.end; w64 += gridDim.x) {
     const uint32_t w = (uint32_t)w64;
     const int r = (int)(w / tps);
     const size_t tile = w - (uint32_t)r * tps;
@@ -427,11 +433,10 @@ struct CopySegs {
 // `count` byte segments; tiles_per_seg is sized for the longest one.
 template <int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_copy_segs(CopySegs t, int count,
-                                                        size_t tiles_per_seg, int aligned) {
+                                                        size_t tiles_per_seg, int aligned, Span span) {
   const uint32_t tps = (uint32_t)tiles_per_seg;
-  const uint64_t total = (uint64_t)count * tps;
   const size_t tile_bytes = (size_t)kThreads * U * 16;
-  for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
+  for (uint64_t w64 = (uint64_t)span.begin + blockIdx.x; w64 < span.end; w64 += gridDim.x) {
     const uint32_t w = (uint32_t)w64;
     const int s = (int)(w / tps);
     const size_t tile = w - (uint32_t)s * tps;
@@ -451,12 +456,11 @@ struct CopyPairs {
 // `count` segments of s1*s2 pieces of pc.len BYTES each (strides in bytes).
 template <int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_copy_pieces(CopyPairs t, int count, Pieces pc,
-                                                          size_t tiles_per_piece, int aligned) {
+                                                          size_t tiles_per_piece, int aligned, Span span) {
   // work items are counted in 32 bits (the host refuses launches beyond 2^32 - 1)
   const uint32_t tpp = (uint32_t)tiles_per_piece;
   const uint32_t per_seg = pc.s1 * pc.s2 * tpp;
-  const uint64_t total = (uint64_t)count * per_seg;
-  for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
+  for (uint64_t w64 = (uint64_t)span.begin + blockIdx.x; w64 < span.end; w64 += gridDim.x) {
     const uint32_t w = (uint32_t)w64;
     const uint32_t s = w / per_seg;
     const uint32_t rem = w - s * per_seg;
@@ -482,12 +486,11 @@ struct GatherArgs {
 // nout / split write streams.
 template <int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_gather_multicast(GatherArgs t, int P, int nout,
-                                                              size_t tiles_per_seg, int split) {
+                                                              size_t tiles_per_seg, int split, Span span) {
   const uint32_t tps = (uint32_t)tiles_per_seg;
-  const uint64_t total = (uint64_t)P * tps * (uint32_t)split;
   const size_t tile_bytes = (size_t)kThreads * U * 16;
   const unsigned tid = threadIdx.x;
-  for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
+  for (uint64_t w64 = (uint64_t)span.begin + blockIdx.x; w64 < span.end; w64 += gridDim.x) {
     const uint32_t w = (uint32_t)w64 / (uint32_t)split;
     const int grp = (int)((uint32_t)w64 - w * (uint32_t)split);
     const int r0 = (int)((long)nout * grp / split), r1 = (int)((long)nout * (grp + 1) / split);
@@ -527,10 +530,9 @@ __global__ __launch_bounds__(kThreads) void k_gather_multicast(GatherArgs t, int
 template <int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_block_transpose(uint8_t* dst, const uint8_t* src,
                                                               size_t rows, size_t cols, size_t m,
-                                                              size_t tiles_per_seg, int aligned) {
+                                                              size_t tiles_per_seg, int aligned, Span span) {
   const uint32_t tps = (uint32_t)tiles_per_seg;
-  const uint64_t total = (uint64_t)rows * cols * tps;
-  for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
+  for (uint64_t w64 = (uint64_t)span.begin + blockIdx.x; w64 < span.end; w64 += gridDim.x) {
     const uint32_t w = (uint32_t)w64;
     const uint32_t blk32 = w / tps;                  // destination block index c*rows + r
     const size_t tile = w - blk32 * tps;
@@ -674,14 +676,13 @@ __device__ __forceinline__ void fold_shards(Load&& load, int k, int g, int first
 template <class Acc, int K, int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int g, int nout,
                                                           size_t n, int first0,
-                                                          size_t tiles_per_seg) {
+                                                          size_t tiles_per_seg, Span span) {
   typedef typename Acc::op Op;
   typedef typename Op::elem elem;
   constexpr int L = Acc::kLanes;
   const uint32_t tps = (uint32_t)tiles_per_seg;
-  const uint64_t total = (uint64_t)nout * tps;
   const unsigned tid = threadIdx.x;
-  for (uint64_t w64 = blockIdx.x; w64 < total; w64 += gridDim.x) {
+  for (uint64_t w64 = (uint64_t)span.begin + blockIdx.x; w64 < span.end; w64 += gridDim.x) {
     const uint32_t w = (uint32_t)w64;
     const int j = (int)(w / tps);
     const size_t tile = w - (uint32_t)j * tps;

@@ -60,6 +60,7 @@ SIGNATURES = {
     "pccl_hip_probe_stream": (_int, [_int, _vp, _sz, _vp]),
     "pccl_hip_set_tuning": (_int, [ctypes.c_char_p, ctypes.c_long]),
     "pccl_hip_get_tuning": (ctypes.c_long, [ctypes.c_char_p]),
+    "pccl_hip_launch_count": (ctypes.c_ulonglong, []),
 }
 
 
@@ -113,6 +114,9 @@ class NativeLib:
 
     def set_tuning(self, key: str, value: int):
         self._check(self._lib.pccl_hip_set_tuning(key.encode(), int(value)))
+
+    def launch_count(self) -> int:
+        return int(self._lib.pccl_hip_launch_count())
 
     def get_tuning(self, key: str) -> int:
         return self._lib.pccl_hip_get_tuning(key.encode())

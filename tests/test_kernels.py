@@ -293,3 +293,52 @@ def test_every_launch_tuning_gives_the_same_bits(target, unroll, nt, grid_cap):
     finally:
         for k, v in saved.items():
             lib.set_tuning(k, v)
+
+
+@pytest.mark.parametrize("launch_mib", [0, 1, 3])
+def test_bounded_launches_give_the_same_bits(target, launch_mib):
+    """A step that goes out as several launches of bounded size (launch_mib)
+    computes what the single launch computes."""
+    import torch
+    from pccl import kernels
+    lib = target.native
+    saved = lib.get_tuning("launch_mib")
+    try:
+        lib.set_tuning("launch_mib", launch_mib)
+        P, B = 4, 150_001
+        for dtype in DTYPES:
+            ins = make_inputs(P, P * B, dtype, seed=23)
+            t_in = [to_torch(x, dtype, target.device) for x in ins]
+            for alg, ref in (("ring", O.ring_reduce_scatter), ("recursive", O.recursive_halving_reduce_scatter)):
+                want = ref(ins, dtype)
+                for mode in ("steps", "fused", "faithful"):
+                    t_out = [torch.zeros(B, dtype=t_in[0].dtype, device=target.device) for _ in range(P)]
+                    kernels.reduce_scatter_ranks(t_out, t_in, alg, mode)
+                    target.sync()
+                    for r in range(P):
+                        assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"{alg}/{mode}/{dtype} rank {r}")
+            g_in = [t[:B + 3] for t in t_in]
+            for alg in ("recursive", "ring"):
+                for mode in ("steps", "fused"):
+                    g_out = [torch.zeros(P * (B + 3), dtype=t_in[0].dtype, device=target.device) for _ in range(P)]
+                    kernels.all_gather_ranks(g_out, g_in, alg, mode)
+                    target.sync()
+                    for r in range(P):
+                        assert_bits_equal(to_numpy(g_out[r], dtype), np.concatenate([x[:B + 3] for x in ins]),
+                                          f"all_gather {alg}/{mode} rank {r}")
+            # 2-D grid and the block transpose
+            want2 = O.reduce_scatter_2d(ins, 2, 2, dtype, "ring")
+            for mode in ("steps", "fused"):
+                t_out = [torch.zeros(B, dtype=t_in[0].dtype, device=target.device) for _ in range(P)]
+                kernels.reduce_scatter_2d_ranks(t_out, t_in, 2, 2, "ring", mode)
+                target.sync()
+                for r in range(P):
+                    assert_bits_equal(to_numpy(t_out[r], dtype), want2[r], f"2d/{mode}/{dtype} rank {r}")
+        src = torch.arange(3 * 5 * 100_003, dtype=torch.int32, device=target.device).view(torch.uint8)
+        dst = torch.zeros_like(src)
+        kernels.block_transpose(dst, src, 3, 5)
+        target.sync()
+        want_t = src.view(torch.int32).view(3, 5, 100_003).transpose(0, 1).reshape(-1)
+        assert torch.equal(dst.view(torch.int32), want_t)
+    finally:
+        lib.set_tuning("launch_mib", saved)
