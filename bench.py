@@ -63,6 +63,9 @@ def parse_args():
                     help="shrink the per-rank message by this factor (1.0 = full size)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true")
+    ap.add_argument("--layout", choices=["auto", "slab", "separate"], default="auto",
+                    help="rank buffers carved from one allocation with a per-rank skew, one allocation each, "
+                         "or (auto) the former from 32 ranks on")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed region launch one plain 1 GiB device copy (k_copy_segs): its "
                          "FETCH_SIZE / WRITE_SIZE readings scale the hardware counters of a rocprofv3 --pmc run")
@@ -75,11 +78,12 @@ def parse_args():
 # workloads: each returns (run_step, info) with inputs resident on the GPU
 # ---------------------------------------------------------------------------
 
-def _randn_bf16(n, std, seed, device):
+def _randn_bf16(n, std, seed, device, out=None):
     import torch
     g = torch.Generator(device=device)
     g.manual_seed(seed)
-    out = torch.empty(n, dtype=torch.bfloat16, device=device)
+    if out is None:
+        out = torch.empty(n, dtype=torch.bfloat16, device=device)
     chunk = 1 << 26
     for i in range(0, n, chunk):      # bounded fp32 temporaries
         m = min(chunk, n - i)
@@ -87,13 +91,38 @@ def _randn_bf16(n, std, seed, device):
     return out
 
 
-def _rand_f32(n, seed, device, uniform=True):
+def _rand_f32(n, seed, device, uniform=True, out=None):
     import torch
     g = torch.Generator(device=device)
     g.manual_seed(seed)
-    if uniform:
-        return torch.rand(n, generator=g, device=device) * 2 - 1
-    return torch.randn(n, generator=g, device=device)
+    if out is None:
+        out = torch.empty(n, dtype=torch.float32, device=device)
+    chunk = 1 << 26
+    for i in range(0, n, chunk):
+        m = min(chunk, n - i)
+        if uniform:
+            out[i:i + m] = torch.rand(m, generator=g, device=device) * 2 - 1
+        else:
+            out[i:i + m] = torch.randn(m, generator=g, device=device)
+    return out
+
+
+LAYOUT = "auto"
+
+
+def _slab(P, numel, dtype, device):
+    """The buffers of P virtual ranks.  'separate': one allocation per rank, what a
+    caller with torch tensors has.  'slab': carved from one allocation with a
+    per-rank skew (pccl.kernels.rank_slab).  'auto': the slab from 32 ranks on,
+    where it measures faster (64 x 1 GiB inputs, fused halving: +8 %), separate
+    allocations below (P = 8: the slab is 2 % slower)."""
+    import torch
+    from pccl import kernels
+    use_slab = LAYOUT == "slab" or (LAYOUT == "auto" and P >= 32)
+    if not use_slab:
+        lens = [numel] * P if isinstance(numel, int) else list(numel)
+        return [torch.empty(n, dtype=dtype, device=device) for n in lens]
+    return kernels.rank_slab(P, numel, dtype, device)
 
 
 def make_ring_rs(P, elems_per_rank, dtype, mode, device, seed=1234, std=1.0):
@@ -101,15 +130,17 @@ def make_ring_rs(P, elems_per_rank, dtype, mode, device, seed=1234, std=1.0):
     from pccl import kernels
     B = elems_per_rank // P
     total = B * P
-    if dtype == "bf16":
-        ins = [_randn_bf16(total, std, seed + r, device) for r in range(P)]
-        es = 2
-    else:
-        ins = [_rand_f32(total, seed + r, device) for r in range(P)]
-        es = 4
-    outs = [torch.empty(B, dtype=ins[0].dtype, device=device) for _ in range(P)]
+    tdt = torch.bfloat16 if dtype == "bf16" else torch.float32
+    ins = _slab(P, total, tdt, device)
+    for r in range(P):
+        if dtype == "bf16":
+            _randn_bf16(total, std, seed + r, device, out=ins[r])
+        else:
+            _rand_f32(total, seed + r, device, out=ins[r])
+    es = 2 if dtype == "bf16" else 4
+    outs = _slab(P, B, tdt, device)
     m = kernels.mode_code(mode)
-    work = [torch.empty_like(ins[r]) for r in range(P)] if m != kernels.MODE_FUSED and P > 2 else None
+    work = _slab(P, total, tdt, device) if m != kernels.MODE_FUSED and P > 2 else None
 
     def step():
         kernels.reduce_scatter_ranks(outs, ins, "ring", m, work)
@@ -118,7 +149,7 @@ def make_ring_rs(P, elems_per_rank, dtype, mode, device, seed=1234, std=1.0):
         # the three execution modes must agree bit for bit
         ref = [torch.empty_like(o) for o in outs]
         other = kernels.MODE_FUSED if m != kernels.MODE_FUSED else kernels.MODE_STEPS
-        w2 = work if work is not None else [torch.empty_like(ins[r]) for r in range(P)]
+        w2 = work if work is not None else _slab(P, total, tdt, device)
         kernels.reduce_scatter_ranks(ref, ins, "ring", other, w2)
         torch.cuda.synchronize()
         return all(torch.equal(a.view(torch.uint8), b.view(torch.uint8)) for a, b in zip(outs, ref))
@@ -150,8 +181,11 @@ def make_rh_pair(count_elems, device, seed=7):
     import torch
     from pccl import _native, kernels
     B = count_elems
-    ins = [_randn_bf16(2 * B, 1.0, seed + r, device) for r in range(2)]
-    work = [t.clone() for t in ins]
+    ins = _slab(2, 2 * B, torch.bfloat16, device)
+    work = _slab(2, 2 * B, torch.bfloat16, device)
+    for r in range(2):
+        _randn_bf16(2 * B, 1.0, seed + r, device, out=ins[r])
+        work[r].copy_(ins[r])
     lib = _native.load()
 
     def step():
@@ -182,10 +216,12 @@ def make_rh_full(P, elems_per_rank, mode, device, seed=21):
     from pccl import kernels
     B = elems_per_rank // P
     total = B * P
-    ins = [_randn_bf16(total, 1.0, seed + r, device) for r in range(P)]
-    outs = [torch.empty(B, dtype=torch.bfloat16, device=device) for _ in range(P)]
+    ins = _slab(P, total, torch.bfloat16, device)
+    for r in range(P):
+        _randn_bf16(total, 1.0, seed + r, device, out=ins[r])
+    outs = _slab(P, B, torch.bfloat16, device)
     m = kernels.mode_code(mode)
-    work = [torch.empty_like(ins[r]) for r in range(P)] if m != kernels.MODE_FUSED else None
+    work = _slab(P, total, torch.bfloat16, device) if m != kernels.MODE_FUSED else None
 
     def step():
         kernels.reduce_scatter_ranks(outs, ins, "recursive", m, work)
@@ -228,11 +264,13 @@ def make_all_gather(P, shard_bytes, mode, device, uneven=False, seed=3):
         lens = [int(n - int(torch.randint(0, n // 8, (1,), generator=g))) for _ in range(P)]
     else:
         lens = [n] * P
-    ins = [_randn_bf16(l, 1.0, seed + r, device) for r, l in enumerate(lens)]
+    ins = _slab(P, lens, torch.bfloat16, device)
+    for r, l in enumerate(lens):
+        _randn_bf16(l, 1.0, seed + r, device, out=ins[r])
     nbytes = [2 * l for l in lens]
     off = kernels.padded_offsets(nbytes, 256) if uneven else [r * shard_bytes for r in range(P)]
     total = off[-1] + (nbytes[-1] + 255) // 256 * 256 if uneven else P * shard_bytes
-    outs = [torch.empty(total // 2, dtype=torch.bfloat16, device=device) for _ in range(P)]
+    outs = _slab(P, total // 2, torch.bfloat16, device)
     m = kernels.mode_code(mode if mode else "fused")
 
     if uneven:
@@ -276,7 +314,9 @@ def make_all_gather(P, shard_bytes, mode, device, uneven=False, seed=3):
 def make_kway(k, n, device, seed=11):
     import torch
     from pccl import kernels
-    shards = [_rand_f32(n, seed + r, device, uniform=False) for r in range(k)]
+    shards = _slab(k, n, torch.float32, device)
+    for r in range(k):
+        _rand_f32(n, seed + r, device, uniform=False, out=shards[r])
     out = torch.empty(n, device=device)
 
     def step():
@@ -509,7 +549,9 @@ def cpu_baseline(info):
 # ---------------------------------------------------------------------------
 
 def main():
+    global LAYOUT
     args = parse_args()
+    LAYOUT = args.layout
     if args.gpus != 1:
         print(f"bench.py: this build runs all virtual ranks on ONE GPU and issues no inter-GPU collective; "
               f"--gpus {args.gpus} is not supported (use --gpus 1).", file=sys.stderr)
@@ -633,7 +675,7 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": info["dtype"], "data": "synthetic",
         "config": {"workload": f"{args.workload}: {info['desc']}", "algorithmic_bytes_per_step": info["alg_bytes"],
                    "launches_per_step": launched, "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
-                   "wall_ms_per_step": round(wall_ms / args.steps, 4), "verified": ok,
+                   "wall_ms_per_step": round(wall_ms / args.steps, 4), "verified": ok, "layout": LAYOUT,
                    "tuning": {k: lib.get_tuning(k) for k in ("grid_cap", "unroll", "unroll_copy", "nt_load", "nt_store", "launch_mib")}},
         "roofline": roof, "cpu_baseline": cpu,
     }

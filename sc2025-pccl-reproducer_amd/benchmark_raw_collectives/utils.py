@@ -9,6 +9,7 @@ timed calls between two device events (benchmark_raw_collectives/utils.py:16-33)
 import os
 
 import torch
+from torch.profiler import record_function
 
 
 def world_size_from_env(default: int = 8) -> int:
@@ -22,15 +23,19 @@ def time_something(comm, fn, *args, warmup_iters=5, timed_iters=20, **kwargs):
     the shared stream between barriers, so every rank gets the same figure."""
     start_event = torch.cuda.Event(enable_timing=True)
     end_event = torch.cuda.Event(enable_timing=True)
-    for _ in range(warmup_iters):
-        fn(*args, **kwargs)
+    # the ranges a torch profiler run shows, named as the reference names them
+    # (benchmark_raw_collectives/utils.py:20,27)
+    for i in range(warmup_iters):
+        with record_function(f"warmup_{i}"):
+            fn(*args, **kwargs)
     comm.Barrier()
     torch.cuda.synchronize()
     if comm.Get_rank() == 0:
         start_event.record()
     comm.Barrier()
-    for _ in range(timed_iters):
-        fn(*args, **kwargs)
+    for i in range(timed_iters):
+        with record_function(f"iteration_{i}"):
+            fn(*args, **kwargs)
     comm.Barrier()
     if comm.Get_rank() == 0:
         end_event.record()

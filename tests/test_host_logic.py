@@ -256,3 +256,24 @@ def test_threads_share_nothing_but_the_rendezvous(cpu):
         P = 2 + i
         for o in res[i]:
             assert torch.equal(o, torch.full((3,), float(P * (P + 1) // 2)))
+
+
+def test_rank_slab_layout():
+    """Buffers of the virtual ranks carved from one allocation: equal strides of
+    the longest buffer (rounded to 256 bytes) plus the skew, no overlap."""
+    import torch
+    from pccl import kernels
+    bufs = kernels.rank_slab(4, [100, 7, 0, 100], torch.bfloat16, "cpu", skew_bytes=512)
+    assert [b.numel() for b in bufs] == [100, 7, 0, 100] and all(b.dtype == torch.bfloat16 for b in bufs)
+    stride = 256 + 512
+    assert bufs[1].data_ptr() - bufs[0].data_ptr() == stride
+    assert bufs[3].data_ptr() - bufs[0].data_ptr() == 3 * stride
+    for r, b in enumerate(bufs):
+        b.fill_(float(r))
+    assert all(bool((b == float(r)).all()) for r, b in enumerate(bufs))
+    same = kernels.rank_slab(3, 64, torch.float32, "cpu", skew_bytes=0)
+    assert same[1].data_ptr() - same[0].data_ptr() == 256
+    with pytest.raises(ValueError):
+        kernels.rank_slab(2, 8, torch.float32, "cpu", skew_bytes=100)
+    with pytest.raises(ValueError):
+        kernels.rank_slab(2, [8], torch.float32, "cpu")
