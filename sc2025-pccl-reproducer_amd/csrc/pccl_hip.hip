@@ -1129,22 +1129,20 @@ int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream) {
   if (nbytes < 4096) return fail(PCCL_HIP_EINVAL, "%s: buffer must hold at least 4096 bytes", what);
   if (!buf || ((uintptr_t)buf & 15u)) return fail(PCCL_HIP_EINVAL, "%s: buffer must be 16-byte aligned", what);
   const size_t nvec = nbytes / 16;
-  const size_t per_tile = (size_t)kThreads * 4;   // vectors per workgroup
+  // vectors per thread: four for the read stream, one for the write stream, the
+  // shapes that sustain the most on MI355X (writes: 6.8 TB/s with 4 KiB per
+  // workgroup against 6.0 with 16 KiB)
+  const size_t per_tile = (size_t)kThreads * (kind == 0 ? 4 : 1);
   const size_t tiles = (nvec + per_tile - 1) / per_tile;
   if (tiles > kMaxGrid) return fail(PCCL_HIP_EINVAL, "%s: buffer too large", what);
   hipStream_t st = (hipStream_t)stream;
-  for_spans(tiles, per_tile * 16, 1, 0, [&](Span span, unsigned) {
-    u32x4* p = (u32x4*)buf + (size_t)span.begin * per_tile;
-    const size_t left = nvec - (size_t)span.begin * per_tile;
-    const size_t cnt = (size_t)(span.end - span.begin) * per_tile;
-    const size_t nv = cnt < left ? cnt : left;
-    if (kind == 0)
-      hipLaunchKernelGGL((k_probe_read<4, true>), dim3(span.end - span.begin), dim3(kThreads), 0, st,
-                         (const u32x4*)p, (u32x4*)buf, nv);
-    else
-      hipLaunchKernelGGL((k_probe_write<4, false>), dim3(span.end - span.begin), dim3(kThreads), 0, st, p, nv,
-                         0x3f803f80u);
-  });
+  if (kind == 0)
+    hipLaunchKernelGGL((k_probe_read<4, true>), dim3((unsigned)tiles), dim3(kThreads), 0, st,
+                       (const u32x4*)buf, (u32x4*)buf, nvec);
+  else
+    hipLaunchKernelGGL((k_probe_write<1, false>), dim3((unsigned)tiles), dim3(kThreads), 0, st, (u32x4*)buf, nvec,
+                       0x3f803f80u);
+  g_launches.fetch_add(1, std::memory_order_relaxed);
   return launch_status(what);
 }
 
