@@ -48,7 +48,7 @@ int launch_status(const char* what) {
 
 std::atomic<long> g_grid_cap{0};
 std::atomic<long> g_unroll{4};        // vectors per thread and operand, add kernels
-std::atomic<long> g_unroll_copy{1};   // ... copy kernels (4 KiB per workgroup: best for the all_gather steps)
+std::atomic<long> g_unroll_copy{2};   // ... copy kernels (two 4 KiB chunks per workgroup, 8 chunks apart: see copy_vec)
 // Unused dynamic LDS requested per workgroup, only to bound how many workgroups
 // share a CU (160 KiB of LDS): the fewer are resident, the narrower the address
 // window the chip streams from at any moment.  0 = as many as fit (8).
@@ -129,6 +129,12 @@ size_t tiles_for(size_t nbytes, int unroll) {
   size_t nvec = nbytes / 16 + 2;
   size_t per = (size_t)kThreads * (size_t)unroll;
   return (nvec + per - 1) / per;
+}
+
+// Tiles of a copy: whole groups of kXcds, which share their chunks (copy_vec).
+size_t copy_tiles_for(size_t nbytes, int unroll) {
+  const size_t t = tiles_for(nbytes, unroll);
+  return unroll > 1 ? (t + kXcds - 1) / kXcds * kXcds : t;
 }
 
 struct Tune {
@@ -248,7 +254,7 @@ int launch_copy(const CopySegs& segs, int count, hipStream_t stream, const char*
   bool aligned = true;
   for (int s = 0; s < count && aligned; ++s)
     aligned = segs.nbytes[s] == 0 || (is16(segs.dst[s]) && is16(segs.src[s]) && (segs.nbytes[s] & 15u) == 0);
-  CopyLaunch l{&segs, count, tiles_for(longest, t.unroll), aligned ? 1 : 0, stream};
+  CopyLaunch l{&segs, count, copy_tiles_for(longest, t.unroll), aligned ? 1 : 0, stream};
   if (int rc = check_work_items((size_t)count, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);
@@ -278,7 +284,7 @@ int launch_copy_pieces(const CopyPairs& segs, int count, const Pieces& pc, hipSt
   chk.b1 = chk.b2 = 0;
   bool aligned = pieces_aligned(chk, 1);
   for (int s = 0; s < count && aligned; ++s) aligned = is16(segs.dst[s]) && is16(segs.src[s]);
-  CopyPiecesLaunch l{&segs, count, pc, tiles_for(pc.len, t.unroll), aligned ? 1 : 0, stream};
+  CopyPiecesLaunch l{&segs, count, pc, copy_tiles_for(pc.len, t.unroll), aligned ? 1 : 0, stream};
   if (int rc = check_work_items((size_t)count * pc.s1 * pc.s2, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);
@@ -648,7 +654,7 @@ int pccl_hip_block_transpose(void* dst, const void* src, size_t rows, size_t col
   Tune t = current_tune(true);
   const bool aligned = is16(dst) && is16(src) && (m_bytes & 15u) == 0;
   TransposeLaunch l{(uint8_t*)dst, (const uint8_t*)src, rows, cols, m_bytes,
-                    tiles_for(m_bytes, t.unroll), aligned ? 1 : 0, (hipStream_t)stream};
+                    copy_tiles_for(m_bytes, t.unroll), aligned ? 1 : 0, (hipStream_t)stream};
   if (rows > kMaxWorkItems || cols > kMaxWorkItems / rows)
     return fail(PCCL_HIP_EINVAL, "%s: rows*cols too large", what);
   if (int rc = check_work_items(rows * cols, l.tiles, what)) return rc;
@@ -684,7 +690,7 @@ int pccl_hip_all_gather_uneven_virtual(void* const* outputs, const void* const* 
   int split = (int)g_gather_split.load(std::memory_order_relaxed);
   if (split <= 0) split = (P + 3) / 4;
   if (split > P) split = P;
-  GatherLaunch l{&args, P, P, split, tiles_for(longest, t.unroll), g_gather_nt.load() != 0,
+  GatherLaunch l{&args, P, P, split, copy_tiles_for(longest, t.unroll), g_gather_nt.load() != 0,
                  (unsigned)g_lds_pad_gather.load(), (hipStream_t)stream};
   if (int rc = check_work_items((size_t)P * (size_t)split, l.tiles, what)) return rc;
   with_tuning(t, l);

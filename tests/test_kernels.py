@@ -342,3 +342,33 @@ def test_bounded_launches_give_the_same_bits(target, launch_mib):
         assert torch.equal(dst.view(torch.int32), want_t)
     finally:
         lib.set_tuning("launch_mib", saved)
+
+
+@pytest.mark.parametrize("unroll", [1, 2, 4, 8])
+def test_copy_chunk_mapping_covers_every_byte(target, unroll):
+    """The vectors of a copying thread come from 4 KiB chunks 8 apart: every
+    length around the boundaries of chunks and of groups of 8 tiles, aligned or
+    not, is copied completely and nothing else is written."""
+    import torch
+    from pccl import kernels
+    lib = target.native
+    saved = lib.get_tuning("unroll_copy")
+    chunk = 4096
+    lengths = sorted({c * chunk + d for c in (0, 1, 7, 8, 9, 15, 16, 17, 8 * unroll - 1, 8 * unroll, 8 * unroll + 1,
+                                              16 * unroll + 3) for d in (-17, -16, -1, 0, 1, 16, 33) if c * chunk + d > 0})
+    try:
+        lib.set_tuning("unroll_copy", unroll)
+        for shift_d, shift_s in ((0, 0), (16, 0), (3, 3), (5, 9)):
+            srcs, dsts, want = [], [], []
+            for i, n in enumerate(lengths):
+                g = torch.Generator().manual_seed(i)
+                s = torch.randint(0, 256, (n + 64,), dtype=torch.uint8, generator=g).to(target.device)
+                d = torch.full((n + 64,), 0xEE, dtype=torch.uint8, device=target.device)
+                srcs.append(s[shift_s:shift_s + n]); dsts.append(d[shift_d:shift_d + n]); want.append((d, s))
+            kernels.copy_batched(dsts, srcs)
+            target.sync()
+            for (d, s), n in zip(want, lengths):
+                assert torch.equal(d[shift_d:shift_d + n], s[shift_s:shift_s + n]), f"length {n} shifts {shift_d},{shift_s}"
+                assert bool((d[:shift_d] == 0xEE).all()) and bool((d[shift_d + n:] == 0xEE).all()), f"length {n}"
+    finally:
+        lib.set_tuning("unroll_copy", saved)
