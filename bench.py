@@ -311,7 +311,9 @@ def make_all_gather(P, shard_bytes, mode, device, uneven=False, seed=3):
     return step, info
 
 
-def make_kway(k, n, device, seed=11):
+def make_kway(k, n, mode, device, seed=11):
+    """k shards folded in ring order from shard 1: in one pass (fused), or as
+    the k-1 per-hop accumulate launches the pass replaces (steps)."""
     import torch
     from pccl import kernels
     # 128 MiB shards: one allocation each measures 2 % faster than the skewed slab
@@ -321,21 +323,41 @@ def make_kway(k, n, device, seed=11):
     for r in range(k):
         _rand_f32(n, seed + r, device, uniform=False, out=shards[r])
     out = torch.empty(n, device=device)
+    per_hop = kernels.mode_code(mode if mode else "fused") != kernels.MODE_FUSED
 
-    def step():
+    def fused():
         kernels.reduce_kway(out, shards, "ring", 1 % k)
 
+    def hops():
+        kernels.add(out, shards[1 % k], shards[2 % k])
+        for t in range(2, k):
+            kernels.accumulate(out, shards[(1 + t) % k])
+
+    step = hops if per_hop else fused
+
     def verify():
+        got = out.clone()
+        (fused if per_hop else hops)()          # the other way must give the same bits
+        torch.cuda.synchronize()
+        if not torch.equal(got.view(torch.int32), out.view(torch.int32)):
+            return False
         m = min(n, 1 << 22)
         acc = shards[1 % k][:m].clone()
         for t in range(1, k):
             acc += shards[(1 + t) % k][:m]
-        return torch.equal(out[:m], acc)
+        return torch.equal(got[:m], acc)
 
-    kb = (k + 1) * n * 4
-    info = dict(alg_bytes=kb, kernel="k_reduce_kway", kernel_bytes=kb, kernel_launches=1, launches=1,
-                desc=f"fused one-pass reduce of {k} fp32 shards of {n} elements ({n * 4 / MiB:.0f} MiB each), "
-                     f"ring order", dtype="f32", P=k, B=n, verify=verify)
+    if per_hop:
+        kb = 3 * n * 4                                       # one hop: 2 reads + 1 write
+        info = dict(alg_bytes=(k - 1) * kb, kernel="k_add_segs", kernel_bytes=kb, kernel_launches=k - 1,
+                    launches=k - 1,
+                    desc=f"reduce of {k} fp32 shards of {n} elements ({n * 4 / MiB:.0f} MiB each) as {k - 1} "
+                         f"per-hop accumulate launches, ring order", dtype="f32", P=k, B=n, verify=verify)
+    else:
+        kb = (k + 1) * n * 4
+        info = dict(alg_bytes=kb, kernel="k_reduce_kway", kernel_bytes=kb, kernel_launches=1, launches=1,
+                    desc=f"fused one-pass reduce of {k} fp32 shards of {n} elements ({n * 4 / MiB:.0f} MiB each), "
+                         f"ring order", dtype="f32", P=k, B=n, verify=verify)
     return step, info
 
 
@@ -355,7 +377,7 @@ def build_workload(name, mode, scale, device):
     if name == "cfg4u":
         return make_all_gather(16, sc(128 * MiB), mode, device, uneven=True)
     if name == "cfg5":
-        return make_kway(32, sc(32 * MiB), device)
+        return make_kway(32, sc(32 * MiB), mode, device)
     raise ValueError(name)
 
 
