@@ -70,7 +70,8 @@ def parse_args():
                     help="after the timed region launch one plain 1 GiB device copy (k_copy_segs): its "
                          "FETCH_SIZE / WRITE_SIZE readings scale the hardware counters of a rocprofv3 --pmc run")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
-                    help="launch tuning of the library (grid_cap, unroll, unroll_copy, nt_load, nt_store)")
+                    help="launch tuning of the library: any key of pccl_hip_set_tuning (grid_cap, unroll, unroll_copy, "
+                         "nt_load, nt_store, lds_pad*, launch_mib, gather_split, unroll_gather, gather_nt)")
     return ap.parse_args()
 
 
