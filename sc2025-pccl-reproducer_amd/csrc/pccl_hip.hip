@@ -103,7 +103,7 @@ unsigned grid_for(size_t total_tiles) {
 // pieces under 0.5 GiB lose again to the drain at the end of every launch.
 // Copies and the multicast gather do not show it; the fused reduce gains 2 %
 // for 8 and 16 shards and loses for 32 (its workgroups live k loads long, and
-// so does the drain), see launch_kway.
+// so does the drain), see KwayLaunch.
 template <class F>
 void for_spans(size_t items, size_t item_bytes, size_t multiple, long target_mib, F&& launch) {
   if (items == 0) return;
@@ -358,6 +358,8 @@ struct KwayLaunch {
     static_assert(U == 1, "the fused reduce is launched with one vector per thread");
 #define PCCL_KWAY(KV) \
   hipLaunchKernelGGL((k_reduce_kway<Acc, KV, U, NTL, NTS>), dim3(grid), dim3(kThreads), lds_pad, stream, *args, k, g, nout, n, first0, tiles, span)
+    // folds over at most 16 shards go out as launches 1.5 times the size of the add kernels' (+2 %);
+    // longer folds lose more to the drain of a launch than they gain, and stay one launch
     for_spans((size_t)nout * tiles, kTileBytes * U * ((size_t)k + 1), 1, k <= 16 ? add_launch_mib() * 3 / 2 : 0, [&](Span span, unsigned grid) {
       if (order == PCCL_HIP_ORDER_RING) { PCCL_KWAY(0); return; }
       switch (k) {
