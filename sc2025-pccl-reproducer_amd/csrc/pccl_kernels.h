@@ -124,6 +124,10 @@ struct AccF32 {
     r.z = __float_as_uint(f[2]); r.w = __float_as_uint(f[3]);
     return r;
   }
+  // one hop on whole input vectors: partial sums can stay in input format
+  static constexpr bool kPacked = true;
+  static __device__ __forceinline__ u32x4 add_vec(u32x4 a, u32x4 b) { return OpF32::add(a, b); }
+  static __device__ __forceinline__ u32x4 settle(u32x4 v) { return v; }
 };
 
 template <bool PER_HOP>
@@ -164,6 +168,25 @@ struct AccBF16 {
     r.z = (bf16_round_hi(f[4]) >> 16) | bf16_round_hi(f[5]);
     r.w = (bf16_round_hi(f[6]) >> 16) | bf16_round_hi(f[7]);
     return r;
+  }
+  // With a rounding per hop every partial sum is a bf16 value again, so partial
+  // sums can stay packed two to a word (half the registers of fp32 lanes).
+  static constexpr bool kPacked = PER_HOP;
+  static __device__ __forceinline__ uint32_t add_word(uint32_t a, uint32_t b) {
+    return cvt_pk_bf16(__uint_as_float(a << 16) + __uint_as_float(b << 16),
+                       __uint_as_float(a & 0xffff0000u) + __uint_as_float(b & 0xffff0000u));
+  }
+  static __device__ __forceinline__ u32x4 add_vec(u32x4 a, u32x4 b) {
+    u32x4 r;
+    r.x = add_word(a.x, b.x); r.y = add_word(a.y, b.y);
+    r.z = add_word(a.z, b.z); r.w = add_word(a.w, b.w);
+    return r;
+  }
+  // the NaN patterns of the packed conversion become the canonical one
+  static __device__ __forceinline__ u32x4 settle(u32x4 v) {
+    float f[8];
+    widen(v, f);
+    return narrow(f);
   }
 };
 
@@ -608,6 +631,45 @@ __device__ __forceinline__ void tree_sum(Load& load, int first, float* out) {
   }
 }
 
+// The same butterfly on whole vectors, G subtrees side by side: vec[r] holds
+// S(r, G), the sum over the leaves m = r (mod G), so a leaf of this tree is the
+// group of G adjacent operands G*b .. G*b+G-1 and load(b, vec) fetches all G.
+// Depth first, a single subtree reads its operands in bit-reversed order
+// (0, K/2, K/4, 3K/4, ...): consecutive loads lie half the operand range apart,
+// which costs 10-15 % of the bandwidth on MI355X (same k and data in natural
+// order: 6.5 TB/s, bit-reversed: 5.6; groups of 4-8 adjacent operands in
+// bit-reversed group order: 6.3-6.6).  The caller finishes with the last
+// log2 G levels, vec[r] += vec[r + h] for h = G/2 .. 1.
+template <class Acc, int KG, int M, int H, int G, class Load>
+__device__ __forceinline__ void tree_vec(Load& load, u32x4* out) {
+  if constexpr (H == KG) {
+    load(M, out);
+  } else {
+    u32x4 lo[G], hi[G];
+    tree_vec<Acc, KG, M, 2 * H, G>(load, lo);
+    tree_vec<Acc, KG, M + H, 2 * H, G>(load, hi);
+#pragma unroll
+    for (int r = 0; r < G; ++r) out[r] = Acc::add_vec(lo[r], hi[r]);
+#if defined(__HIP_DEVICE_COMPILE__)
+    // After every pair of leaf groups: the sums must exist here (an empty asm
+    // takes them as operands) and nothing moves across.  Left alone, the
+    // scheduler issues all K loads first and sinks the adds to the end: every
+    // loaded vector stays live (up to 256 VGPRs, one wave per SIMD).  With the
+    // fence 2*G loads are in flight.
+    if constexpr (2 * H == KG) {
+#pragma unroll
+      for (int r = 0; r < G; ++r) asm volatile("" : "+v"(out[r]));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#endif
+  }
+}
+
+// Subtrees evaluated side by side for a butterfly over K >= 16 operands (measured:
+// 8 for K = 64 and 32, 4 or 8 alike for K = 16; K = 8 is faster depth first).
+template <int K>
+constexpr int tree_group() { return K >= 32 ? 8 : 4; }
+
 // Left fold over `count` operands in cyclic order first, first+1, ...
 // load(q, f) fills the L fp32 lanes of operand q; acc receives the result.
 // Folds over kFoldPairedFrom or more operands issue their loads two at a time
@@ -713,11 +775,40 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const size_t v = base + (size_t)u * kThreads + tid;
+      // an address is a workgroup-uniform 64-bit base plus a 32-bit lane offset:
+      // the unrolled folds then need no vector registers for their k addresses
+      const size_t wg_byte = eoff * sizeof(elem) + (base + (size_t)u * kThreads) * 16;
+      const uint32_t lane_byte = tid * 16u;
+      if constexpr (K >= 16 && Acc::kPacked) {
+        if (v < nvec) {
+          constexpr int G = tree_group<K>();
+          u32x4 part[G];
+          auto group_load = [&](int b, u32x4* x) {
+#pragma unroll
+            for (int r = 0; r < G; ++r) {
+              int q = first ^ (G * b + r);
+#if defined(__HIP_DEVICE_COMPILE__)
+              // ties the fetch of the shard pointer to this place: left alone, all K
+              // pointers are fetched up front and spill out of the scalar registers
+              asm volatile("" : "+s"(q));
+#endif
+              x[r] = ld16<NTL>((const u32x4*)((const uint8_t*)t.shard[q] + wg_byte + lane_byte));
+            }
+          };
+          tree_vec<Acc, K / G, 0, 1, G>(group_load, part);
+#pragma unroll
+          for (int h = G / 2; h >= 1; h /= 2) {
+#pragma unroll
+            for (int r = 0; r < h; ++r) part[r] = Acc::add_vec(part[r], part[r + h]);
+          }
+          st16<NTS>((u32x4*)out + v, Acc::settle(part[0]));
+        }
+      } else
       if (v < nvec) {
         float acc[L];
         fold_shards<Acc, K, L>(
             [&](int q, float* f) {
-              Acc::widen(ld16<NTL>((const u32x4*)((const elem*)t.shard[q] + eoff) + v), f);
+              Acc::widen(ld16<NTL>((const u32x4*)((const uint8_t*)t.shard[q] + wg_byte + lane_byte)), f);
             },
             k, g, first, first_outer, acc);
         st16<NTS>((u32x4*)out + v, Acc::narrow(acc));
@@ -738,6 +829,9 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
       float acc1[1];
       fold_shards<Acc, K, 1>(
           [&](int q, float* f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+            if constexpr (K > 0) asm volatile("" : "+s"(q));   // fetch the pointer here, see group_load
+#endif
             elem e = ((const elem*)t.shard[q] + eoff)[i];
             if constexpr (sizeof(elem) == 4) f[0] = e;
             else f[0] = __uint_as_float((uint32_t)e << 16);
