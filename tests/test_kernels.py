@@ -372,3 +372,56 @@ def test_copy_chunk_mapping_covers_every_byte(target, unroll):
                 assert bool((d[:shift_d] == 0xEE).all()) and bool((d[shift_d + n:] == 0xEE).all()), f"length {n}"
     finally:
         lib.set_tuning("unroll_copy", saved)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("k,order", [(8, "ring"), (16, "ring"), (8, "halving"), (16, "halving"), (32, "halving"),
+                                     (64, "halving")])
+def test_reduce_kway_special_values(target, dtype, k, order):
+    """Infinities, NaNs of any payload, signed zeros, denormals and the largest
+    finite values folded by the fused reduce give the oracle's bits in every
+    code path (fp32 lanes, packed bf16 partial sums)."""
+    import torch
+    rng = np.random.default_rng(99 + k)
+    n = 5000
+    if dtype == O.F32:
+        pool = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 3.4e38, -3.4e38, 1e-38,
+                         1.0 + 2 ** -23, 2 ** -24, 16777216.0, 0.5, -0.25], dtype=np.float32)
+        shards = [rng.choice(pool, n, p=None).astype(np.float32) for _ in range(k)]
+        # mostly ordinary values, so that specials meet finite partial sums as well
+        for s in shards:
+            keep = rng.random(n) < 0.9
+            s[keep] = rng.standard_normal(int(keep.sum())).astype(np.float32)
+    else:
+        pool = np.array([0x0000, 0x8000, 0x3F80, 0xBF80, 0x7F80, 0xFF80, 0x7FC0, 0x7FA1, 0xFFFF, 0x0001, 0x8001,
+                         0x7F7F, 0xFF7F, 0x0080, 0x3F81, 0x3B80, 0x4B80, 0x3FFF], dtype=np.uint16)
+        shards = [rng.choice(pool, n).astype(np.uint16) for _ in range(k)]
+        for s in shards:
+            keep = rng.random(n) < 0.9
+            s[keep] = O.f32_to_bf16(rng.standard_normal(int(keep.sum())).astype(np.float32))
+    first = 5 % k
+    ts = [to_torch(x, dtype, target.device) for x in shards]
+    out = torch.zeros_like(ts[0])
+    target.native.reduce_kway(out.data_ptr(), [t.data_ptr() for t in ts], n, CODE[dtype],
+                              0 if order == "ring" else 1, first, True, target.stream())
+    target.sync()
+    with np.errstate(all="ignore"):
+        if order == "ring":
+            want = shards[first]
+            for t in range(1, k):
+                want = O.vector_add(want, shards[(first + t) % k], dtype)
+        else:
+            v = [shards[first ^ m] for m in range(k)]
+            h = k // 2
+            while h >= 1:
+                for m in range(h):
+                    v[m] = O.vector_add(v[m], v[m + h], dtype)
+                h //= 2
+            want = v[0]
+    got = to_numpy(out, dtype)
+    if dtype == O.F32:
+        # which payload and sign a sum of two different NaNs carries is left open by
+        # IEEE 754 and differs between processors: NaN must meet NaN, all else bit for bit
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        got, want = np.where(np.isnan(got), np.float32(0), got), np.where(np.isnan(want), np.float32(0), want)
+    assert_bits_equal(got, want, "reduce_kway special values")
