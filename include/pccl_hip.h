@@ -271,7 +271,9 @@ int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream);
  * key: "grid_cap" (max workgroups per launch, 0 = one tile per workgroup),
  *      "unroll"   (128-bit vectors per thread per operand of the add kernels:
  *                  1, 2, 4 or 8), "unroll_copy" (the same for the copy kernels),
- *      "nt_load" / "nt_store" (0/1: non-temporal global loads / stores),
+ *      "nt_load" / "nt_store" (non-temporal global loads / stores: 1 always,
+ *                  0 never, -1, the default: for calls whose footprint exceeds
+ *                  the Infinity Cache and the L2s, 288 MiB),
  *      "lds_pad" / "lds_pad_copy" / "lds_pad_kway" / "lds_pad_gather" (bytes of
  *                  unused LDS per workgroup, 0..65536: bounds the workgroups
  *                  resident per CU; lds_pad_kway = -1, the default, lets the
@@ -280,7 +282,7 @@ int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream);
  *      "gather_split"  (workgroups sharing one shard tile of the multicast
  *                  gather, each storing to 1/gather_split of the outputs;
  *                  0, the default = four outputs per workgroup),
- *      "gather_nt" (0/1: non-temporal stores in the multicast gather),
+ *      "gather_nt" (non-temporal stores in the multicast gather: 1, 0 or -1 as above),
  *      "launch_mib" (a step of the add kernels goes out as equal launches that
  *                  move about this many MiB each, a fused reduce over at most
  *                  16 shards as launches 1.5 times as large; 0 = always one
