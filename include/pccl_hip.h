@@ -198,6 +198,33 @@ int pccl_hip_reduce_scatter_virtual(void* const* outputs,
                                     int dtype, const char* algorithm, int mode,
                                     void* stream);
 
+/* The per-step reduce_scatter (PCCL_HIP_MODE_STEPS of the call above, same
+ * schedules, same bits) for callers that cannot allocate device memory and have
+ * no workspace to pass: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference (its shim
+ * allocates the work buffers as torch tensors on every call,
+ * pccl/src/pccl.cpp:58-59,71-73).  The work buffers live in an array that is
+ * part of the library's code object: PCCL_HIP_NOALLOC_SCRATCH_BYTES of device
+ * memory on every GPU the library is used on, held until the process ends.
+ * The call allocates and frees nothing, on the device or on the host.
+ *   limit : P <= PCCL_HIP_MAX_RANKS, and P slices of P*B elements, each rounded
+ *           up to 256 bytes, must fit PCCL_HIP_NOALLOC_SCRATCH_BYTES; larger
+ *           shapes are refused with PCCL_HIP_EINVAL (use the call above with
+ *           caller-owned work buffers).
+ *   set-up: the first call on a device looks the array's address up
+ *           (hipGetSymbolAddress) with that device current; make it outside
+ *           graph capture.  Later calls only enqueue.
+ *   sharing: every call on a GPU uses that GPU's one array, so calls that can
+ *           overlap on one GPU (different streams, different threads) race;
+ *           calls on one stream are ordered and safe.  Nothing has to be
+ *           cleared between calls: every scratch element a call reads has been
+ *           written earlier in the same call. */
+#define PCCL_HIP_NOALLOC_SCRATCH_BYTES (32u * 1024u * 1024u)
+int pccl_hip_reduce_scatter_virtual_noalloc(void* const* outputs,
+                                            const void* const* inputs, int P,
+                                            size_t B, int dtype,
+                                            const char* algorithm, void* stream);
+
 /* all_gather over P virtual ranks, in bytes.  Replaces all_gather_mpi
  * (pccl/src/pccl.cpp:87-142) and recursiveDoublingAllGatherGPU
  * (pccl/src/all_gather.cpp:15-69).

@@ -437,7 +437,28 @@ int launch_kway(const KwayArgs& args, int k, int g, int nout, size_t n, int dtyp
 // does not matter.
 struct AddTriple { void* dst; const void* a; const void* b; };
 
-int launch_add_list(const std::vector<AddTriple>& list, size_t n, int dtype, hipStream_t stream,
+// One entry per virtual rank: on the stack up to the ranks of one launch (so a
+// collective over at most PCCL_HIP_MAX_RANKS ranks touches no heap either), on
+// the host heap beyond.
+template <class T>
+class RankList {
+ public:
+  explicit RankList(size_t n) : n_(n), p_(small_) {
+    if (n > (size_t)kMaxSeg) { big_.resize(n); p_ = big_.data(); }
+  }
+  RankList(const RankList&) = delete;
+  RankList& operator=(const RankList&) = delete;
+  T& operator[](size_t i) { return p_[i]; }
+  const T& operator[](size_t i) const { return p_[i]; }
+  size_t size() const { return n_; }
+ private:
+  size_t n_;
+  T* p_;
+  T small_[kMaxSeg];
+  std::vector<T> big_;
+};
+
+int launch_add_list(const RankList<AddTriple>& list, size_t n, int dtype, hipStream_t stream,
                     const char* what) {
   for (size_t i0 = 0; i0 < list.size(); i0 += kMaxSeg) {
     const int cnt = (int)(list.size() - i0 < (size_t)kMaxSeg ? list.size() - i0 : (size_t)kMaxSeg);
@@ -450,7 +471,7 @@ int launch_add_list(const std::vector<AddTriple>& list, size_t n, int dtype, hip
 
 struct CopyItem { void* dst; const void* src; size_t nbytes; };
 
-int launch_copy_list(const std::vector<CopyItem>& list, hipStream_t stream, const char* what) {
+int launch_copy_list(const RankList<CopyItem>& list, hipStream_t stream, const char* what) {
   for (size_t i0 = 0; i0 < list.size(); i0 += kMaxSeg) {
     const int cnt = (int)(list.size() - i0 < (size_t)kMaxSeg ? list.size() - i0 : (size_t)kMaxSeg);
     CopySegs segs;
@@ -724,10 +745,13 @@ int pccl_hip_all_gather_uneven_virtual(void* const* outputs, const void* const* 
   return launch_status(what);
 }
 
-int pccl_hip_reduce_scatter_virtual(void* const* outputs, const void* const* inputs,
-                                    void* const* work, int P, size_t B, int dtype,
-                                    const char* algorithm, int mode, void* stream) {
-  const char* what = "pccl_hip_reduce_scatter_virtual";
+}  // extern "C"
+
+namespace {
+
+// The argument checks of a reduce_scatter over virtual ranks, before anything touches the device.
+int check_reduce_scatter_args(void* const* outputs, const void* const* inputs, int P, int dtype,
+                              const char* algorithm, int mode, const char* what) {
   if (int rc = check_dtype(dtype, what)) return rc;
   if (!algorithm) return fail(PCCL_HIP_EINVAL, "%s: algorithm is NULL", what);
   const bool ring = !strcmp(algorithm, "ring");
@@ -740,11 +764,20 @@ int pccl_hip_reduce_scatter_virtual(void* const* outputs, const void* const* inp
     return fail(PCCL_HIP_EINVAL, "%s: recursive halving needs a power-of-two P, got %d", what, P);
   if (mode != PCCL_HIP_MODE_STEPS && mode != PCCL_HIP_MODE_FUSED && mode != PCCL_HIP_MODE_FAITHFUL)
     return fail(PCCL_HIP_EINVAL, "%s: unknown mode %d", what, mode);
+  if (int rc = check_table((const void* const*)outputs, P, what, "outputs")) return rc;
+  if (int rc = check_table(inputs, P, what, "inputs")) return rc;
+  return PCCL_HIP_OK;
+}
+
+// reduce_scatter over P virtual ranks; `what` names the entry point in messages.
+int reduce_scatter_ranks(void* const* outputs, const void* const* inputs, void* const* work, int P,
+                         size_t B, int dtype, const char* algorithm, int mode, void* stream,
+                         const char* what) {
+  if (int rc = check_reduce_scatter_args(outputs, inputs, P, dtype, algorithm, mode, what)) return rc;
+  const bool ring = !strcmp(algorithm, "ring");
   if (mode == PCCL_HIP_MODE_FUSED && P > kMaxSeg)
     return fail(PCCL_HIP_EINVAL, "%s: the fused mode folds at most %d ranks in one launch, got P = %d", what,
                 kMaxSeg, P);
-  if (int rc = check_table((const void* const*)outputs, P, what, "outputs")) return rc;
-  if (int rc = check_table(inputs, P, what, "inputs")) return rc;
   const bool need_work = (mode == PCCL_HIP_MODE_FAITHFUL && P > 1) || (mode == PCCL_HIP_MODE_STEPS && P > 2);
   if (need_work) if (int rc = check_table((const void* const*)work, P, what, "work")) return rc;
   if (B == 0) return PCCL_HIP_OK;
@@ -768,7 +801,7 @@ int pccl_hip_reduce_scatter_virtual(void* const* outputs, const void* const* inp
   }
 
   const bool faithful = mode == PCCL_HIP_MODE_FAITHFUL;
-  std::vector<CopyItem> copies((size_t)P);
+  RankList<CopyItem> copies((size_t)P);
   if (faithful) {  // buf <- input
     for (int r = 0; r < P; ++r) copies[r] = CopyItem{work[r], inputs[r], (size_t)P * B * es};
     if (int rc = launch_copy_list(copies, st, what)) return rc;
@@ -778,7 +811,7 @@ int pccl_hip_reduce_scatter_virtual(void* const* outputs, const void* const* inp
       copies[r] = CopyItem{outputs[r], (const uint8_t*)work[r] + (size_t)r * B * es, B * es};
     return launch_copy_list(copies, st, what);
   };
-  std::vector<AddTriple> adds((size_t)P);
+  RankList<AddTriple> adds((size_t)P);
 
   if (ring) {
     for (int step = 0; step < P - 1; ++step) {
@@ -831,6 +864,74 @@ int pccl_hip_reduce_scatter_virtual(void* const* outputs, const void* const* inp
   return faithful ? copy_out() : PCCL_HIP_OK;
 }
 
+// Work buffers of pccl_hip_reduce_scatter_virtual_noalloc: one array per GPU,
+// part of the loaded code object, held until the process ends.  `scratch` is a
+// host-side stand-in for the symbol; the address of a device's copy comes from
+// hipGetSymbolAddress with that device current and is kept per device.
+constexpr size_t kScratchBytes = PCCL_HIP_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+int scratch_of_current_device(void** out, const char* what) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(PCCL_HIP_ENODEV, "%s: hipGetDevice failed: %s", what, hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(PCCL_HIP_ENODEV, "%s: device index %d outside [0, %d)", what, dev, kMaxDevices);
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return fail(PCCL_HIP_ENODEV, "%s: hipGetSymbolAddress(scratch) failed on device %d: %s", what, dev,
+                  hipGetErrorString(e));
+    g_scratch_ptr[dev].store(p, std::memory_order_release);   // two threads racing here store the same address
+  }
+  *out = p;
+  return PCCL_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int pccl_hip_reduce_scatter_virtual(void* const* outputs, const void* const* inputs,
+                                    void* const* work, int P, size_t B, int dtype,
+                                    const char* algorithm, int mode, void* stream) {
+  return reduce_scatter_ranks(outputs, inputs, work, P, B, dtype, algorithm, mode, stream,
+                              "pccl_hip_reduce_scatter_virtual");
+}
+
+int pccl_hip_reduce_scatter_virtual_noalloc(void* const* outputs, const void* const* inputs, int P,
+                                            size_t B, int dtype, const char* algorithm, void* stream) {
+  const char* what = "pccl_hip_reduce_scatter_virtual_noalloc";
+  if (int rc = check_dtype(dtype, what)) return rc;
+  if (P < 1 || P > kMaxSeg)
+    return fail(PCCL_HIP_EINVAL, "%s: P = %d outside [1, %d]", what, P, kMaxSeg);
+  // rank r works in scratch[r * slice, (r + 1) * slice), slice = P*B elements rounded up to 256 bytes
+  const size_t es = esize_of(dtype);
+  if (B > kScratchBytes / es / (size_t)P)
+    return fail(PCCL_HIP_EINVAL, "%s: P = %d ranks of %zu elements need more than the %zu bytes of built-in scratch",
+                what, P, B, kScratchBytes);
+  const size_t slice = ((size_t)P * B * es + 255) / 256 * 256;
+  if (slice * (size_t)P > kScratchBytes)
+    return fail(PCCL_HIP_EINVAL,
+                "%s: work buffers of %d ranks x %zu bytes exceed the %zu bytes of built-in scratch; "
+                "use pccl_hip_reduce_scatter_virtual with caller-owned work buffers",
+                what, P, slice, kScratchBytes);
+  if (int rc = check_reduce_scatter_args(outputs, inputs, P, dtype, algorithm, PCCL_HIP_MODE_STEPS, what)) return rc;
+  if (B == 0) return PCCL_HIP_OK;
+  void* work[kMaxSeg];
+  const bool need_work = P > 2;   // the per-step mode needs no work buffers for one or two ranks
+  if (need_work) {
+    void* base = nullptr;
+    if (int rc = scratch_of_current_device(&base, what)) return rc;
+    for (int r = 0; r < P; ++r) work[r] = (uint8_t*)base + (size_t)r * slice;
+  }
+  return reduce_scatter_ranks(outputs, inputs, need_work ? work : nullptr, P, B, dtype, algorithm,
+                              PCCL_HIP_MODE_STEPS, stream, what);
+}
+
 int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs, int P,
                                 size_t block_bytes, const char* algorithm, int mode, void* stream) {
   const char* what = "pccl_hip_all_gather_virtual";
@@ -861,7 +962,7 @@ int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs,
   }
 
   // out[r][r] <- in[r]   (pccl/src/all_gather.cpp:31-35)
-  std::vector<CopyItem> c((size_t)P);
+  RankList<CopyItem> c((size_t)P);
   for (int r = 0; r < P; ++r)
     c[r] = CopyItem{(uint8_t*)outputs[r] + (size_t)r * block_bytes, inputs[r], block_bytes};
   if (int rc = launch_copy_list(c, st, what)) return rc;

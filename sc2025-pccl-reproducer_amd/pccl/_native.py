@@ -27,6 +27,7 @@ MODE_FAITHFUL = 2
 
 MAX_RANKS = 64            # per launch / fused modes / 2-D grids
 MAX_VIRTUAL_RANKS = 4096  # per-step modes of the 1-D collectives
+NOALLOC_SCRATCH_BYTES = 32 << 20   # built-in work space of reduce_scatter_virtual_noalloc
 ABI_VERSION = 1
 
 LIB_NAME = "libpccl_hip.so"
@@ -52,6 +53,7 @@ SIGNATURES = {
     "pccl_hip_gather_place": (_int, [_vp, _vpp, _szp, _szp, _int, _vp]),
     "pccl_hip_block_transpose": (_int, [_vp, _vp, _sz, _sz, _sz, _vp]),
     "pccl_hip_reduce_scatter_virtual": (_int, [_vpp, _vpp, _vpp, _int, _sz, _int, ctypes.c_char_p, _int, _vp]),
+    "pccl_hip_reduce_scatter_virtual_noalloc": (_int, [_vpp, _vpp, _int, _sz, _int, ctypes.c_char_p, _vp]),
     "pccl_hip_all_gather_virtual": (_int, [_vpp, _vpp, _int, _sz, ctypes.c_char_p, _int, _vp]),
     "pccl_hip_all_gather_uneven_virtual": (_int, [_vpp, _vpp, _szp, _szp, _int, _vp]),
     "pccl_hip_reduce_scatter_2d_virtual": (_int, [_vpp, _vpp, _vpp, _vpp, _int, _int, _sz, _int, ctypes.c_char_p,
@@ -160,6 +162,11 @@ class NativeLib:
         self._check(self._lib.pccl_hip_reduce_scatter_virtual(
             _ptr_table(outputs), _ptr_table(inputs), _ptr_table(work), P, B, dtype,
             algorithm.encode(), mode, stream))
+
+    def reduce_scatter_virtual_noalloc(self, outputs, inputs, B, dtype, algorithm, stream=0):
+        """Per-step reduce_scatter whose work buffers are the library's built-in scratch."""
+        self._check(self._lib.pccl_hip_reduce_scatter_virtual_noalloc(
+            _ptr_table(outputs), _ptr_table(inputs), len(inputs), B, dtype, algorithm.encode(), stream))
 
     def all_gather_virtual(self, outputs, inputs, block_bytes, algorithm, mode=MODE_STEPS, stream=0):
         P = len(inputs)

@@ -27,6 +27,12 @@ constexpr hipError_t hipSuccess = 0;
 inline hipError_t hipGetLastError() { return hipSuccess; }
 inline const char* hipGetErrorString(hipError_t) { return "emulated"; }
 
+// a "device" array is ordinary host memory here; its symbol is its address
+#define __align__(n) __attribute__((aligned(n)))
+#define HIP_SYMBOL(x) (x)
+inline hipError_t hipGetDevice(int* dev) { *dev = 0; return hipSuccess; }
+inline hipError_t hipGetSymbolAddress(void** ptr, const void* symbol) { *ptr = const_cast<void*>(symbol); return hipSuccess; }
+
 inline uint32_t __float_as_uint(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }
 inline float __uint_as_float(uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; }
 
