@@ -303,13 +303,21 @@ int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream);
  *                  the Infinity Cache and the L2s, 288 MiB),
  *      "lds_pad" / "lds_pad_copy" / "lds_pad_kway" / "lds_pad_gather" (bytes of
  *                  unused LDS per workgroup, 0..65536: bounds the workgroups
- *                  resident per CU; lds_pad_kway = -1, the default, lets the
- *                  fused reduce choose),
- *      "unroll_gather" (vectors per thread of the multicast gather: 1, 2, 4, 8),
- *      "gather_split"  (workgroups sharing one shard tile of the multicast
- *                  gather, each storing to 1/gather_split of the outputs;
+ *                  resident per CU; -1, the default of lds_pad_kway and
+ *                  lds_pad_gather, lets the launch choose),
+ *      "unroll_gather" (vectors per thread of the all_gather placement kernels:
+ *                  1, 2, 4, 8; 0, the default: one in the multicast kernel,
+ *                  four in the time-blocked one),
+ *      "gather_strip"  (fused all_gather: work items per XCD and strip of the
+ *                  time-blocked kernel, in which an XCD walks a strip of its
+ *                  tiles once per output; 0 = the multicast kernel, in which a
+ *                  workgroup stores its tile to several outputs at once; -1, the
+ *                  default: time-blocked, 160, for shards of at least
+ *                  "gather_strip_from" bytes, default 2 MiB),
+ *      "gather_split"  (multicast kernel: workgroups sharing one shard tile,
+ *                  each storing to 1/gather_split of the outputs;
  *                  0, the default = four outputs per workgroup),
- *      "gather_nt" (non-temporal stores in the multicast gather: 1, 0 or -1 as above),
+ *      "gather_nt" (non-temporal stores in both kernels: 1, 0 or -1 as above),
  *      "launch_mib" (a step of the add kernels goes out as equal launches that
  *                  move about this many MiB each, a fused reduce over at most
  *                  16 shards as launches 1.5 times as large; 0 = always one

@@ -55,10 +55,12 @@ std::atomic<long> g_unroll_copy{2};   // ... copy kernels (two 4 KiB chunks per 
 std::atomic<long> g_lds_pad{0};        // add kernels
 std::atomic<long> g_lds_pad_copy{0};   // copy kernels
 std::atomic<long> g_lds_pad_kway{-1};  // fused reduce; -1 = chosen per launch (see launch_kway)
-std::atomic<long> g_lds_pad_gather{0}; // multicast gather
+std::atomic<long> g_lds_pad_gather{-1}; // all_gather placement kernels; -1 = chosen per launch
 std::atomic<long> g_gather_split{0};   // groups of outputs per shard tile in the multicast gather; 0 = four outputs a group
 std::atomic<long> g_gather_nt{-1};     // non-temporal stores in the multicast gather (-1: by footprint, like nt_store)
-std::atomic<long> g_unroll_gather{1};  // vectors per thread in the multicast gather
+std::atomic<long> g_unroll_gather{0};  // vectors per thread in the all_gather placement kernels; 0 = chosen per launch
+std::atomic<long> g_gather_strip{-1};  // work items per XCD and strip of the time-blocked gather; 0 = the multicast kernel, -1 = chosen per launch
+std::atomic<long> g_gather_strip_from{-1};  // shortest longest-shard (bytes) the time-blocked gather is chosen for when gather_strip = -1
 std::atomic<unsigned long long> g_launches{0};   // kernel launches issued so far
 std::atomic<long> g_launch_mib{1024};  // traffic per launch of the add kernels, MiB (0 = a step is one launch whatever its size)
 // Non-temporal loads / stores: 1 = always, 0 = never, -1 = by the footprint of
@@ -69,6 +71,8 @@ std::atomic<long> g_launch_mib{1024};  // traffic per launch of the add kernels,
 std::atomic<long> g_nt_load{-1};
 std::atomic<long> g_nt_store{-1};
 constexpr size_t kStreamFrom = (size_t)288 << 20;   // 256 MiB Infinity Cache + 8 x 4 MiB L2
+constexpr long kStripItems = 160;                   // work items per XCD and strip of the time-blocked gather
+constexpr long kStripFrom = 2 << 20;                // ... chosen for shards of at least this many bytes
 
 // Footprint of the collective being launched (inputs, work buffers and outputs of
 // all ranks), set by the collective entry points; 0 inside a plain kernel call,
@@ -528,14 +532,19 @@ int pccl_hip_set_tuning(const char* key, long value) {
       return fail(PCCL_HIP_EINVAL, "set_tuning: %s must be in [%ld, 65536]", key, lowest);
     (!strcmp(key, "lds_pad") ? g_lds_pad : !strcmp(key, "lds_pad_copy") ? g_lds_pad_copy : g_lds_pad_kway) = value;
   } else if (!strcmp(key, "lds_pad_gather")) {
-    if (value < 0 || value > 65536) return fail(PCCL_HIP_EINVAL, "set_tuning: lds_pad_gather must be in [0, 65536]");
+    if (value < -1 || value > 65536) return fail(PCCL_HIP_EINVAL, "set_tuning: lds_pad_gather must be in [-1, 65536]");
     g_lds_pad_gather = value;
   } else if (!strcmp(key, "gather_split")) {
     if (value < 0 || value > kMaxSeg) return fail(PCCL_HIP_EINVAL, "set_tuning: gather_split must be in [0, %d]", kMaxSeg);
     g_gather_split = value;
+  } else if (!strcmp(key, "gather_strip")) {
+    if (value < -1 || value > 65536) return fail(PCCL_HIP_EINVAL, "set_tuning: gather_strip must be in [-1, 65536]");
+    g_gather_strip = value;
+  } else if (!strcmp(key, "gather_strip_from")) {
+    g_gather_strip_from = value < 0 ? -1 : value;
   } else if (!strcmp(key, "unroll_gather")) {
-    if (value != 1 && value != 2 && value != 4 && value != 8)
-      return fail(PCCL_HIP_EINVAL, "set_tuning: unroll_gather must be 1, 2, 4 or 8");
+    if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8)
+      return fail(PCCL_HIP_EINVAL, "set_tuning: unroll_gather must be 0, 1, 2, 4 or 8");
     g_unroll_gather = value;
   } else if (!strcmp(key, "launch_mib")) {
     if (value < 0) return fail(PCCL_HIP_EINVAL, "set_tuning: launch_mib must be >= 0");
@@ -563,6 +572,8 @@ long pccl_hip_get_tuning(const char* key) {
   if (!strcmp(key, "lds_pad_gather")) return g_lds_pad_gather;
   if (!strcmp(key, "gather_split")) return g_gather_split;
   if (!strcmp(key, "unroll_gather")) return g_unroll_gather;
+  if (!strcmp(key, "gather_strip")) return g_gather_strip;
+  if (!strcmp(key, "gather_strip_from")) return g_gather_strip_from;
   if (!strcmp(key, "gather_nt")) return g_gather_nt;
   if (!strcmp(key, "launch_mib")) return g_launch_mib;
   if (!strcmp(key, "nt_load")) return g_nt_load;
@@ -728,7 +739,54 @@ int pccl_hip_all_gather_uneven_virtual(void* const* outputs, const void* const* 
   if (longest == 0) return PCCL_HIP_OK;
   const size_t moved = ((size_t)P + 1) * payload;   // every shard read, and written to P outputs
   Tune t = current_tune(false, moved);
-  t.unroll = (int)g_unroll_gather.load(std::memory_order_relaxed);
+  // Two kernels.  Time-blocked strips (k_gather_strips): an XCD walks a strip of
+  // its tiles once per output, so it feeds one write stream at a time and re-reads
+  // the strip from its L2.  Measured on MI355X against the multicast kernel below
+  // (shards of 8 ... 512 MiB, 4 ... 64 ranks): +9 ... +15 %; 16 shards of 128 MiB
+  // 5.85 -> 6.75 TB/s.  Four tiles per workgroup (with one the kernel is bound by
+  // the latency of its load, 5.4 TB/s); strips of 160 work items = 2.5 MiB per XCD
+  // (beyond the 4 MiB of an L2 the re-reads miss: 3.7 TB/s); three workgroups per
+  // CU (48 KiB of unused LDS each, +1 %).  A strip that divides the shard exactly
+  // is 5-15 % slower than one a quarter longer (the two outputs an XCD writes
+  // around a change of output then lie a power of two apart), so short shards get
+  // strips a quarter longer than their work items.
+  long strip = g_gather_strip.load(std::memory_order_relaxed);
+  if (strip < 0) {
+    long from = g_gather_strip_from.load(std::memory_order_relaxed);
+    if (from < 0) from = kStripFrom;
+    strip = (P >= 2 && longest >= (size_t)from) ? kStripItems : 0;
+  }
+  const long unroll_set = g_unroll_gather.load(std::memory_order_relaxed);
+  const long pad_set = g_lds_pad_gather.load(std::memory_order_relaxed);
+  t.unroll = unroll_set > 0 ? (int)unroll_set : strip > 0 ? 4 : 1;
+  const unsigned lds = (unsigned)(pad_set >= 0 ? pad_set : strip > 0 ? 49152 : 0);
+  if (strip > 0) {
+    const int U = t.unroll;
+    // work items per shard and XCD, each U tiles; whole strips
+    const size_t items = (tiles_for(longest, 1) + kXcds * U - 1) / (kXcds * U);
+    if (g_gather_strip.load(std::memory_order_relaxed) < 0 && items + items / 4 + 1 < (size_t)strip)
+      strip = (long)(items + items / 4 + 1);
+    const size_t n_local = (items + (size_t)strip - 1) / (size_t)strip * (size_t)strip;
+    if (int rc = check_work_items((size_t)P * (size_t)P * kXcds, n_local, what)) return rc;
+    const bool nts = stream_hint(g_gather_nt.load(), moved);
+    hipStream_t st = (hipStream_t)stream;
+#define PCCL_STRIPS(UV)                                                                                              \
+  case UV:                                                                                                          \
+    if (nts) hipLaunchKernelGGL((k_gather_strips<UV, false, true>), dim3(grid), dim3(kThreads), lds, st, args, P, P, (uint32_t)n_local, (uint32_t)strip, span); \
+    else hipLaunchKernelGGL((k_gather_strips<UV, false, false>), dim3(grid), dim3(kThreads), lds, st, args, P, P, (uint32_t)n_local, (uint32_t)strip, span);    \
+    break;
+    for_spans((size_t)P * (size_t)P * kXcds * n_local, 0, 1, 0, [&](Span span, unsigned grid) {
+      switch (U) {
+        PCCL_STRIPS(1)
+        PCCL_STRIPS(2)
+        PCCL_STRIPS(8)
+        default:
+        PCCL_STRIPS(4)
+      }
+    });
+#undef PCCL_STRIPS
+    return launch_status(what);
+  }
   // A workgroup holds one 4 KiB tile of a shard and stores it into four of the
   // P outputs; the P/4 workgroups of a tile are launched side by side, so all but
   // the first find the tile in cache.  Measured on MI355X against one workgroup
@@ -739,7 +797,7 @@ int pccl_hip_all_gather_uneven_virtual(void* const* outputs, const void* const* 
   if (split <= 0) split = (P + 3) / 4;
   if (split > P) split = P;
   GatherLaunch l{&args, P, P, split, copy_tiles_for(longest, t.unroll), stream_hint(g_gather_nt.load(), moved),
-                 (unsigned)g_lds_pad_gather.load(), (hipStream_t)stream};
+                 lds, (hipStream_t)stream};
   if (int rc = check_work_items((size_t)P * (size_t)split, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);

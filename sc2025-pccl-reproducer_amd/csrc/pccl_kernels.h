@@ -560,6 +560,61 @@ __global__ __launch_bounds__(kThreads) void k_gather_multicast(GatherArgs t, int
   }
 }
 
+// The same placement, blocked in time: workgroup w runs on XCD w % 8 (workgroups
+// are dealt to the dies round robin), and the workgroups of one XCD, taken in
+// index order, walk a strip of `strip` of that XCD's 4 KiB tiles of shard k once
+// per output: first the whole strip into output 0, then the same strip into
+// output 1, ...  At any moment an XCD therefore feeds one write stream (two
+// around a change of output) instead of nout, and every pass after the first
+// finds the strip in that XCD's L2.  XCD x owns the tiles t = x (mod 8) of every
+// shard, as in copy_vec.  n_local = tiles per shard and XCD, a multiple of strip.
+template <int U, bool NTL, bool NTS>
+__global__ __launch_bounds__(kThreads) void k_gather_strips(GatherArgs t, int P, int nout, uint32_t n_local,
+                                                           uint32_t strip, Span span) {
+  // a work item moves U of its XCD's tiles (8 tiles apart in the shard); n_local and strip count work items
+  const unsigned tid = threadIdx.x;
+  const uint32_t per_shard = n_local * (uint32_t)nout;
+  const uint32_t per_strip = strip * (uint32_t)nout;
+  for (uint64_t w64 = (uint64_t)span.begin + blockIdx.x; w64 < span.end; w64 += gridDim.x) {
+    const uint32_t w = (uint32_t)w64;
+    const uint32_t x = w % (uint32_t)kXcds, seq = w / (uint32_t)kXcds;
+    const uint32_t k = seq / per_shard;
+    uint32_t rem = seq - k * per_shard;
+    const uint32_t s = rem / per_strip;
+    rem -= s * per_strip;
+    const uint32_t r = rem / strip;
+    const size_t tile0 = (size_t)(s * strip + (rem - r * strip)) * (kXcds * U) + x;   // then tile0 + 8, + 16, ...
+    const size_t nb = t.nbytes[k];
+    if (tile0 != 0 && tile0 * kTileBytes >= nb + 16) continue;
+    const uint8_t* src = (const uint8_t*)t.ins[k];
+    uint8_t* dst = (uint8_t*)t.outs[r] + t.dst_off[k];
+    const size_t nvec = nb / 16;
+    if (((((uintptr_t)src) | ((uintptr_t)dst)) & 15u) == 0) {
+      const size_t v0 = tile0 * kThreads + tid;
+      if (v0 + (size_t)(U - 1) * kXcds * kThreads < nvec) {
+        u32x4 xv[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) xv[j] = ld16<NTL>((const u32x4*)src + v0 + (size_t)j * kXcds * kThreads);
+#pragma unroll
+        for (int j = 0; j < U; ++j) st16<NTS>((u32x4*)dst + v0 + (size_t)j * kXcds * kThreads, xv[j]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+          const size_t v = v0 + (size_t)j * kXcds * kThreads;
+          if (v < nvec) st16<NTS>((u32x4*)dst + v, ld16<NTL>((const u32x4*)src + v));
+        }
+      }
+      if (tile0 == 0 && tid < nb - nvec * 16) dst[nvec * 16 + tid] = src[nvec * 16 + tid];   // the last nb % 16 bytes
+    } else {
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const size_t tile = tile0 + (size_t)j * kXcds;
+        if (tile == 0 || tile * kTileBytes < nb + 16) copy_tile<1, NTL, NTS>(dst, src, nb, tile);
+      }
+    }
+  }
+}
+
 // dst[c][r][0:m] = src[r][c][0:m] (bytes): the 2-D block transpose.
 template <int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_block_transpose(uint8_t* dst, const uint8_t* src,

@@ -172,16 +172,17 @@ def test_all_gather_uneven_padded_to_256(target):
 
 
 @pytest.mark.parametrize("P", [1, 3, 5, 16])
-@pytest.mark.parametrize("split", [0, 1, 2, 3, 64])
+@pytest.mark.parametrize("split,strip", [(0, 0), (1, 0), (2, 0), (3, 0), (64, 0), (0, 1), (0, 2), (0, 256), (0, -1)])
 @pytest.mark.parametrize("unroll,nt", [(1, 1), (4, 0)])
-def test_multicast_gather_tunings_give_the_same_bytes(target, P, split, unroll, nt):
+def test_multicast_gather_tunings_give_the_same_bytes(target, P, split, strip, unroll, nt):
     """However the outputs of a shard tile are shared among workgroups
-    (gather_split), the gathered bytes are the same; ragged lengths and odd
+    (gather_split), or walked strip by strip and output by output
+    (gather_strip), the gathered bytes are the same; ragged lengths and odd
     rank counts included."""
     import torch
     from pccl import kernels
     lib = target.native
-    keys = ("gather_split", "unroll_gather", "gather_nt")
+    keys = ("gather_split", "unroll_gather", "gather_nt", "gather_strip", "gather_strip_from")
     saved = {k: lib.get_tuning(k) for k in keys}
     rng = np.random.default_rng(100 + P)
     nbytes = [int(x) for x in rng.integers(0, 30_000, P)]
@@ -191,6 +192,8 @@ def test_multicast_gather_tunings_give_the_same_bytes(target, P, split, unroll, 
     total = off[-1] + nbytes[-1] + 7
     try:
         lib.set_tuning("gather_split", split)
+        lib.set_tuning("gather_strip", strip)
+        lib.set_tuning("gather_strip_from", 0)      # strip = -1: the automatic choice, also for these short shards
         lib.set_tuning("unroll_gather", unroll)
         lib.set_tuning("gather_nt", nt)
         t_out = [torch.full((total,), 0x5A, dtype=torch.uint8, device=target.device) for _ in range(P)]
