@@ -7,12 +7,20 @@ Prints ONE JSON line.  A "step" is one whole collective over the virtual ranks
 of the workload with all inputs already resident in HBM; `value` is the
 algorithmic bytes of that collective divided by its time (GB/s, 1 GB = 1e9 B).
 Timing follows benchmark_raw_collectives/utils.py:16-33 of the reference:
-warm-up calls, then the mean over the timed calls between two device events.
+warm-up calls, then the mean over the timed calls between two device events
+recorded on the stream the library launches on.
 
-Workloads (`cfg2` is the one the headline metric is quoted on):
+With no --workload the headline is `cfg2` in the per-step mode (the
+configuration the metric is quoted on: the per-hop accumulate kernel), and
+`config.workloads` carries one row for every other configuration and mode, each
+timed the same way, each with its roofline fraction and a `verified` flag that
+comes from a closed form recomputed with torch (never from a second run of the
+library); `config.latency_us`, `config.ceilings` and `config.drop_in` follow.
+
+Workloads:
   cfg1  ring reduce_scatter, P=4, fp32, 16 Mi elements per rank
   cfg2  ring reduce_scatter, P=8, bf16, 256 Mi elements per rank, per-hop
-        accumulate with bf16 rounding at every hop              (default)
+        accumulate with bf16 rounding at every hop
   cfg3  recursive-halving round at its largest shape: a pair of ranks adding
         512 MiB strided halves (bf16), i.e. round 0 of P=64 with 1 GiB per rank
   cfg3full  the whole recursive-halving reduce_scatter over P=64 resident ranks,
@@ -20,12 +28,12 @@ Workloads (`cfg2` is the one the headline metric is quoted on):
   cfg4  all_gather placement, P=16, bf16 shards of 128 MiB into 2 GiB outputs
   cfg4u the same with uneven shards padded to 256 bytes
   cfg5  fused one-pass reduce of 32 fp32 shards of 32 Mi elements
-  ceilings  what the device sustains for plain streams of 1 GiB: read-only,
-        write-only, copy and 2-reads-1-write add (the practical roofline)
-  sweep  GB/s against message size, 64 MiB .. 2 GiB per operand: accumulate
-        (bf16 and fp32), copy, and the fused 8-way reduce
-  latency  small messages, 4 KiB .. 1 MiB in bf16: microseconds per accumulate,
-        per copy and per whole P=8 ring reduce_scatter (per-step and fused)
+  ceilings  what the device sustains for plain streams of 1 GiB (read-only,
+        write-only, copy, add) and for read:write mixes with no data flowing
+        from the loads to the stores (2:1, 8:1, 32:1, 1:16)
+  sweep  GB/s against message size, 64 MiB .. 2 GiB per operand
+  latency  small messages, 4 KiB .. 1 MiB in bf16: microseconds per call
+  all   (default) cfg2/steps as the headline plus every row above
 
 The CPU baseline (the reference's per-rank algorithm on host cores, one process
 per rank over MPI_Sendrecv, or fork+shared memory where no MPI launcher
@@ -35,6 +43,7 @@ a baseline, not a target.
 from __future__ import annotations
 
 import argparse
+import hashlib
 import json
 import os
 import shutil
@@ -49,16 +58,22 @@ METRIC = "reduce/copy kernel HBM GB/s and % of MI355X peak at 64MB-2GB messages"
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
 MiB = 1 << 20
 
+WORKLOADS = ["cfg1", "cfg2", "cfg3", "cfg3full", "cfg4", "cfg4u", "cfg5"]
+# every (workload, mode) row of the default run besides the headline cfg2/steps
+ALL_ROWS = [("cfg1", "steps"), ("cfg1", "fused"), ("cfg2", "fused"), ("cfg3", "steps"),
+            ("cfg3full", "steps"), ("cfg3full", "fused"), ("cfg4", "steps"), ("cfg4", "fused"),
+            ("cfg4u", "fused"), ("cfg5", "fused"), ("cfg5", "steps")]
+
 
 def parse_args():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="cfg2",
-                    choices=["cfg1", "cfg2", "cfg3", "cfg3full", "cfg4", "cfg4u", "cfg5", "latency", "ceilings", "sweep"])
+    ap.add_argument("--workload", default="all", choices=["all"] + WORKLOADS + ["latency", "ceilings", "sweep"])
     ap.add_argument("--mode", default=None, choices=["steps", "fused", "faithful"],
-                    help="execution mode of the collective (default: per-step replay)")
+                    help="execution mode of the collective (default: per-step replay for the reductions, "
+                         "one fused launch for cfg4, cfg4u and cfg5)")
     ap.add_argument("--scale", type=float, default=1.0,
                     help="shrink the per-rank message by this factor (1.0 = full size)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -71,12 +86,13 @@ def parse_args():
                          "FETCH_SIZE / WRITE_SIZE readings scale the hardware counters of a rocprofv3 --pmc run")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="launch tuning of the library: any key of pccl_hip_set_tuning (grid_cap, unroll, unroll_copy, "
-                         "nt_load, nt_store, lds_pad*, launch_mib, gather_split, unroll_gather, gather_nt)")
+                         "nt_load, nt_store, lds_pad*, launch_mib, gather_strip, gather_split, unroll_gather, gather_nt)")
     return ap.parse_args()
 
 
 # ---------------------------------------------------------------------------
-# workloads: each returns (run_step, info) with inputs resident on the GPU
+# workloads: each builder returns {mode: (run_step, info)} on shared inputs
+# resident on the GPU
 # ---------------------------------------------------------------------------
 
 def _randn_bf16(n, std, seed, device, out=None):
@@ -126,7 +142,34 @@ def _slab(P, numel, dtype, device):
     return kernels.rank_slab(P, numel, dtype, device)
 
 
-def make_ring_rs(P, elems_per_rank, dtype, mode, device, seed=1234, std=1.0):
+def _mode_name(m):
+    return {0: "steps", 1: "fused", 2: "faithful"}[m]
+
+
+def _windows(n, width=1 << 20):
+    """Element windows of a block that a closed form is recomputed on: its first
+    and its last `width` elements (the whole block if it is shorter)."""
+    if n <= 2 * width:
+        return [(0, n)]
+    return [(0, width), (n - width, n)]
+
+
+def _hop(acc, x):
+    """One hop of the reference's accumulate on torch tensors: an IEEE fp32 add,
+    rounded to bfloat16 (nearest even) when the data is bfloat16."""
+    import torch
+    if acc.dtype == torch.bfloat16:
+        return (acc.float() + x.float()).to(torch.bfloat16)
+    return acc + x
+
+
+def _same_bits(a, b):
+    import torch
+    it = torch.int16 if a.dtype == torch.bfloat16 else torch.int32
+    return torch.equal(a.view(it), b.view(it))
+
+
+def make_ring_rs(P, elems_per_rank, dtype, modes, device, seed=1234, std=1.0):
     import torch
     from pccl import kernels
     B = elems_per_rank // P
@@ -140,40 +183,48 @@ def make_ring_rs(P, elems_per_rank, dtype, mode, device, seed=1234, std=1.0):
             _rand_f32(total, seed + r, device, out=ins[r])
     es = 2 if dtype == "bf16" else 4
     outs = _slab(P, B, tdt, device)
-    m = kernels.mode_code(mode)
-    work = _slab(P, total, tdt, device) if m != kernels.MODE_FUSED and P > 2 else None
-
-    def step():
-        kernels.reduce_scatter_ranks(outs, ins, "ring", m, work)
+    shared = {}
 
     def verify():
-        # the three execution modes must agree bit for bit
-        ref = [torch.empty_like(o) for o in outs]
-        other = kernels.MODE_FUSED if m != kernels.MODE_FUSED else kernels.MODE_STEPS
-        w2 = work if work is not None else _slab(P, total, tdt, device)
-        kernels.reduce_scatter_ranks(ref, ins, "ring", other, w2)
+        # closed form of the ring: block j is the left fold over ranks j+1, j+2, ..., j
+        # (pccl/src/reduce_scatter.cpp:127-146), one rounding per hop
         torch.cuda.synchronize()
-        return all(torch.equal(a.view(torch.uint8), b.view(torch.uint8)) for a, b in zip(outs, ref))
+        for j in sorted({0, P // 2, P - 1}):
+            for lo, hi in _windows(B):
+                acc = ins[(j + 1) % P][j * B + lo:j * B + hi]
+                for t in range(2, P + 1):
+                    acc = _hop(acc, ins[(j + t) % P][j * B + lo:j * B + hi])
+                if not _same_bits(outs[j][lo:hi], acc):
+                    return False
+        return True
 
-    launches = {kernels.MODE_STEPS: P - 1, kernels.MODE_FUSED: 1, kernels.MODE_FAITHFUL: P + 1}[m]
-    if m == kernels.MODE_FUSED:
-        kernel_bytes = (P * P + P) * B * es             # reads every input once, writes every output
-        alg_bytes = kernel_bytes
-        kernel = "k_reduce_kway"
-    else:
-        kernel_bytes = 3 * P * B * es                   # one batched step: 2 reads + 1 write per rank
-        alg_bytes = (P - 1) * kernel_bytes
-        kernel = "k_add_segs"
-    info = dict(alg_bytes=alg_bytes, kernel=kernel, kernel_bytes=kernel_bytes,
-                kernel_launches=(P - 1 if m != kernels.MODE_FUSED else 1), launches=launches,
-                desc=f"ring reduce_scatter, P={P} virtual ranks, {dtype}, {total} elements per rank "
-                     f"({total * es / MiB:.0f} MiB), block {B} elements, mode={_mode_name(m)}",
-                dtype=dtype, P=P, B=B, verify=verify)
-    return step, info
+    out = {}
+    for mode in modes:
+        m = kernels.mode_code(mode)
+        if m != kernels.MODE_FUSED and P > 2 and "work" not in shared:
+            shared["work"] = _slab(P, total, tdt, device)
+        work = shared.get("work") if m != kernels.MODE_FUSED else None
 
+        def step(m=m, work=work):
+            kernels.reduce_scatter_ranks(outs, ins, "ring", m, work)
 
-def _mode_name(m):
-    return {0: "steps", 1: "fused", 2: "faithful"}[m]
+        launches = {kernels.MODE_STEPS: P - 1, kernels.MODE_FUSED: 1, kernels.MODE_FAITHFUL: P + 1}[m]
+        if m == kernels.MODE_FUSED:
+            kernel_bytes = (P * P + P) * B * es             # reads every input once, writes every output
+            alg_bytes = kernel_bytes
+            kernel = "k_reduce_kway"
+        else:
+            kernel_bytes = 3 * P * B * es                   # one batched step: 2 reads + 1 write per rank
+            alg_bytes = (P - 1) * kernel_bytes
+            kernel = "k_add_segs"
+        out[mode] = (step, dict(
+            alg_bytes=alg_bytes, kernel=kernel, kernel_bytes=kernel_bytes,
+            kernel_launches=(P - 1 if m != kernels.MODE_FUSED else 1), launches=launches,
+            desc=f"ring reduce_scatter, P={P} virtual ranks, {dtype}, {total} elements per rank "
+                 f"({total * es / MiB:.0f} MiB), block {B} elements, mode={_mode_name(m)}",
+            dtype=dtype, P=P, B=B, verify=verify,
+            verify_how="left fold from rank j+1 recomputed with torch on windows of blocks 0, P/2, P-1"))
+    return out
 
 
 def make_rh_pair(count_elems, device, seed=7):
@@ -198,20 +249,23 @@ def make_rh_pair(count_elems, device, seed=7):
             w.copy_(i)
         step()
         torch.cuda.synchronize()
-        n = min(B, 1 << 24)
-        lo = (ins[0][:n].float() + ins[1][:n].float()).bfloat16()
-        hi = (ins[1][B:B + n].float() + ins[0][B:B + n].float()).bfloat16()
-        return torch.equal(work[0][:n], lo) and torch.equal(work[1][B:B + n], hi)
+        for lo, hi in _windows(B, 1 << 23):
+            low = _hop(ins[0][lo:hi], ins[1][lo:hi])
+            high = _hop(ins[1][B + lo:B + hi], ins[0][B + lo:B + hi])
+            if not (_same_bits(work[0][lo:hi], low) and _same_bits(work[1][B + lo:B + hi], high)):
+                return False
+        return True
 
     kb = 2 * 3 * B * 2
     info = dict(alg_bytes=kb, kernel="k_rh_round", kernel_bytes=kb, kernel_launches=1, launches=1,
                 desc=f"recursive-halving round, one pair of ranks, bf16, halves of {B * 2 / MiB:.0f} MiB "
                      f"(round 0 of P=64 with {4 * B / MiB:.0f} MiB per rank)",
-                dtype="bf16", P=2, B=B, verify=verify)
-    return step, info
+                dtype="bf16", P=2, B=B, verify=verify,
+                verify_how="lower and upper half sums recomputed with torch on windows")
+    return {"steps": (step, info)}
 
 
-def make_rh_full(P, elems_per_rank, mode, device, seed=21):
+def make_rh_full(P, elems_per_rank, modes, device, seed=21):
     """Recursive-halving reduce_scatter with all P ranks resident."""
     import torch
     from pccl import kernels
@@ -221,44 +275,55 @@ def make_rh_full(P, elems_per_rank, mode, device, seed=21):
     for r in range(P):
         _randn_bf16(total, 1.0, seed + r, device, out=ins[r])
     outs = _slab(P, B, torch.bfloat16, device)
-    m = kernels.mode_code(mode)
-    work = _slab(P, total, torch.bfloat16, device) if m != kernels.MODE_FUSED else None
-
-    def step():
-        kernels.reduce_scatter_ranks(outs, ins, "recursive", m, work)
+    shared = {}
 
     def verify():
-        # the halving order of block 0 and block P-1 recomputed with torch on a window
-        n = min(B, 1 << 20)
+        # the halving order of block 0 and block P-1 recomputed with torch on windows
+        torch.cuda.synchronize()
         for j in (0, P - 1):
-            v = [ins[j ^ q][j * B:j * B + n].float() for q in range(P)]
-            h = P // 2
-            while h >= 1:
-                for q in range(h):
-                    v[q] = (v[q] + v[q + h]).bfloat16().float()
-                h //= 2
-            if not torch.equal(outs[j][:n].float(), v[0]):
-                return False
+            for lo, hi in _windows(B, 1 << 19):
+                v = [ins[j ^ q][j * B + lo:j * B + hi] for q in range(P)]
+                h = P // 2
+                while h >= 1:
+                    for q in range(h):
+                        v[q] = _hop(v[q], v[q + h])
+                    h //= 2
+                if not _same_bits(outs[j][lo:hi], v[0]):
+                    return False
         return True
 
     rounds = P.bit_length() - 1
-    if m == kernels.MODE_FUSED:
-        kb = (P * P + P) * B * 2
-        alg, kernel, kl, launches = kb, "k_reduce_kway", 1, 1
-    else:
-        # round r adds (P / 2^(r+1)) blocks per rank: 2 reads + 1 write per element
-        alg = sum(3 * P * (P >> (r + 1)) * B * 2 for r in range(rounds))
-        kb, kernel, kl, launches = alg, "k_rh_round", 1, rounds
-    info = dict(alg_bytes=alg, kernel=kernel, kernel_bytes=kb, kernel_launches=kl, launches=launches,
-                desc=f"recursive-halving reduce_scatter, P={P} resident virtual ranks, bf16, {total} elements per "
-                     f"rank ({total * 2 / MiB:.0f} MiB), {rounds} rounds, mode={_mode_name(m)}",
-                dtype="bf16", P=P, B=B, verify=verify)
-    return step, info
+    out = {}
+    for mode in modes:
+        m = kernels.mode_code(mode)
+        if m != kernels.MODE_FUSED and "work" not in shared:
+            shared["work"] = _slab(P, total, torch.bfloat16, device)
+        work = shared.get("work") if m != kernels.MODE_FUSED else None
+
+        def step(m=m, work=work):
+            kernels.reduce_scatter_ranks(outs, ins, "recursive", m, work)
+
+        if m == kernels.MODE_FUSED:
+            kb = (P * P + P) * B * 2
+            alg, kernel, kl, launches = kb, "k_reduce_kway", 1, 1
+        else:
+            # round r adds (P / 2^(r+1)) blocks per rank: 2 reads + 1 write per element
+            alg = sum(3 * P * (P >> (r + 1)) * B * 2 for r in range(rounds))
+            kb, kernel, kl, launches = alg, "k_rh_round", 1, rounds
+        out[mode] = (step, dict(
+            alg_bytes=alg, kernel=kernel, kernel_bytes=kb, kernel_launches=kl, launches=launches,
+            desc=f"recursive-halving reduce_scatter, P={P} resident virtual ranks, bf16, {total} elements per "
+                 f"rank ({total * 2 / MiB:.0f} MiB), {rounds} rounds, mode={_mode_name(m)}",
+            dtype="bf16", P=P, B=B, verify=verify,
+            verify_how="XOR butterfly of blocks 0 and P-1 recomputed with torch on windows"))
+    return out
 
 
-def make_all_gather(P, shard_bytes, mode, device, uneven=False, seed=3):
+def make_all_gather(P, shard_bytes, modes, device, uneven=False, seed=3):
     import torch
-    from pccl import kernels
+    from pccl import _native, kernels
+    if isinstance(modes, str) or modes is None:      # a single mode: return its (step, info)
+        return make_all_gather(P, shard_bytes, [modes or "fused"], device, uneven, seed)[modes or "fused"]
     n = shard_bytes // 2
     if uneven:
         g = torch.Generator().manual_seed(seed)
@@ -272,21 +337,11 @@ def make_all_gather(P, shard_bytes, mode, device, uneven=False, seed=3):
     off = kernels.padded_offsets(nbytes, 256) if uneven else [r * shard_bytes for r in range(P)]
     total = off[-1] + (nbytes[-1] + 255) // 256 * 256 if uneven else P * shard_bytes
     outs = _slab(P, total // 2, torch.bfloat16, device)
-    m = kernels.mode_code(mode if mode else "fused")
-
-    if uneven:
-        def step():
-            kernels.all_gather_uneven_ranks(outs, ins, off)
-        launches, kernel = 1, "k_gather_multicast"
-    else:
-        def step():
-            kernels.all_gather_ranks(outs, ins, "ring", m)
-        launches = 1 if m == kernels.MODE_FUSED else P
-        kernel = "k_gather_multicast" if m == kernels.MODE_FUSED else "k_copy_segs"
 
     def verify():
+        torch.cuda.synchronize()
         cat = torch.cat([t.view(torch.uint8) for t in ins]) if not uneven else None
-        for o in (outs[0], outs[P - 1]):
+        for o in (outs[0], outs[P // 2], outs[P - 1]):
             ob = o.view(torch.uint8)
             if uneven:
                 for k in range(P):
@@ -297,22 +352,40 @@ def make_all_gather(P, shard_bytes, mode, device, uneven=False, seed=3):
         return True
 
     payload = sum(nbytes)
-    if kernel == "k_gather_multicast":
-        # every shard is read once and written into each of the P outputs
-        alg = (1 + P) * payload
-        kb, kl = alg, 1
-    else:
-        alg = 2 * payload * P                   # 2 * bytes per materialised output, P outputs
-        kb, kl = 2 * P * shard_bytes, P         # one batched step moves one shard per rank
-    info = dict(alg_bytes=alg, kernel=kernel, kernel_bytes=kb, kernel_launches=kl, launches=launches,
-                desc=f"all_gather placement, P={P} virtual ranks, bf16 shards of ~{shard_bytes / MiB:.0f} MiB"
-                     f"{' (uneven, padded to 256 B)' if uneven else ''} into {total / MiB:.0f} MiB outputs, "
-                     f"all {P} outputs materialised, mode={_mode_name(m) if not uneven else 'fused'}",
-                dtype="bf16", P=P, B=n, verify=verify)
-    return step, info
+    out = {}
+    for mode in modes:
+        m = kernels.mode_code(mode if mode else "fused")
+        # the fused placement is the time-blocked kernel from 2 MiB shards on, the multicast kernel below
+        strips = _native.load().get_tuning("gather_strip") != 0 and max(nbytes) >= (
+            max(_native.load().get_tuning("gather_strip_from"), 0) or 2 * MiB)
+        gather_kernel = "k_gather_strips" if strips else "k_gather_multicast"
+        if uneven:
+            def step():
+                kernels.all_gather_uneven_ranks(outs, ins, off)
+            launches, kernel = 1, gather_kernel
+        else:
+            def step(m=m):
+                kernels.all_gather_ranks(outs, ins, "ring", m)
+            launches = 1 if m == kernels.MODE_FUSED else P
+            kernel = gather_kernel if m == kernels.MODE_FUSED else "k_copy_segs"
+        if kernel == gather_kernel:
+            # every shard is read once and written into each of the P outputs
+            alg = (1 + P) * payload
+            kb, kl = alg, 1
+        else:
+            alg = 2 * payload * P                   # 2 * bytes per materialised output, P outputs
+            kb, kl = 2 * P * shard_bytes, P         # one batched step moves one shard per rank
+        out[mode] = (step, dict(
+            alg_bytes=alg, kernel=kernel, kernel_bytes=kb, kernel_launches=kl, launches=launches,
+            desc=f"all_gather placement, P={P} virtual ranks, bf16 shards of ~{shard_bytes / MiB:.0f} MiB"
+                 f"{' (uneven, padded to 256 B)' if uneven else ''} into {total / MiB:.0f} MiB outputs, "
+                 f"all {P} outputs materialised, mode={_mode_name(m) if not uneven else 'fused'}",
+            dtype="bf16", P=P, B=n, verify=verify,
+            verify_how="outputs 0, P/2, P-1 byte-equal to the concatenation of the shards (torch.cat)"))
+    return out
 
 
-def make_kway(k, n, mode, device, seed=11):
+def make_kway(k, n, modes, device, seed=11):
     """k shards folded in ring order from shard 1: in one pass (fused), or as
     the k-1 per-hop accumulate launches the pass replaces (steps)."""
     import torch
@@ -323,67 +396,166 @@ def make_kway(k, n, mode, device, seed=11):
         [torch.empty(n, dtype=torch.float32, device=device) for _ in range(k)]
     for r in range(k):
         _rand_f32(n, seed + r, device, uniform=False, out=shards[r])
-    out = torch.empty(n, device=device)
-    per_hop = kernels.mode_code(mode if mode else "fused") != kernels.MODE_FUSED
+    out_t = torch.empty(n, device=device)
 
     def fused():
-        kernels.reduce_kway(out, shards, "ring", 1 % k)
+        kernels.reduce_kway(out_t, shards, "ring", 1 % k)
 
     def hops():
-        kernels.add(out, shards[1 % k], shards[2 % k])
+        kernels.add(out_t, shards[1 % k], shards[2 % k])
         for t in range(2, k):
-            kernels.accumulate(out, shards[(1 + t) % k])
-
-    step = hops if per_hop else fused
+            kernels.accumulate(out_t, shards[(1 + t) % k])
 
     def verify():
-        got = out.clone()
-        (fused if per_hop else hops)()          # the other way must give the same bits
         torch.cuda.synchronize()
-        if not torch.equal(got.view(torch.int32), out.view(torch.int32)):
-            return False
-        m = min(n, 1 << 22)
-        acc = shards[1 % k][:m].clone()
-        for t in range(1, k):
-            acc += shards[(1 + t) % k][:m]
-        return torch.equal(got[:m], acc)
+        for lo, hi in _windows(n, 1 << 21):
+            acc = shards[1 % k][lo:hi].clone()
+            for t in range(1, k):
+                acc += shards[(1 + t) % k][lo:hi]
+            if not _same_bits(out_t[lo:hi], acc):
+                return False
+        return True
 
-    if per_hop:
-        kb = 3 * n * 4                                       # one hop: 2 reads + 1 write
-        info = dict(alg_bytes=(k - 1) * kb, kernel="k_add_segs", kernel_bytes=kb, kernel_launches=k - 1,
-                    launches=k - 1,
-                    desc=f"reduce of {k} fp32 shards of {n} elements ({n * 4 / MiB:.0f} MiB each) as {k - 1} "
-                         f"per-hop accumulate launches, ring order", dtype="f32", P=k, B=n, verify=verify)
-    else:
-        kb = (k + 1) * n * 4
-        info = dict(alg_bytes=kb, kernel="k_reduce_kway", kernel_bytes=kb, kernel_launches=1, launches=1,
-                    desc=f"fused one-pass reduce of {k} fp32 shards of {n} elements ({n * 4 / MiB:.0f} MiB each), "
-                         f"ring order", dtype="f32", P=k, B=n, verify=verify)
-    return step, info
+    out = {}
+    for mode in modes:
+        per_hop = kernels.mode_code(mode if mode else "fused") != kernels.MODE_FUSED
+        if per_hop:
+            kb = 3 * n * 4                                       # one hop: 2 reads + 1 write
+            info = dict(alg_bytes=(k - 1) * kb, kernel="k_add_segs", kernel_bytes=kb, kernel_launches=k - 1,
+                        launches=k - 1,
+                        desc=f"reduce of {k} fp32 shards of {n} elements ({n * 4 / MiB:.0f} MiB each) as {k - 1} "
+                             f"per-hop accumulate launches, ring order", dtype="f32", P=k, B=n, verify=verify)
+        else:
+            kb = (k + 1) * n * 4
+            info = dict(alg_bytes=kb, kernel="k_reduce_kway", kernel_bytes=kb, kernel_launches=1, launches=1,
+                        desc=f"fused one-pass reduce of {k} fp32 shards of {n} elements ({n * 4 / MiB:.0f} MiB each), "
+                             f"ring order", dtype="f32", P=k, B=n, verify=verify)
+        info["verify_how"] = "left fold from shard 1 recomputed with torch fp32 adds on windows"
+        out[mode] = (hops if per_hop else fused, info)
+    return out
 
 
-def build_workload(name, mode, scale, device):
+def default_mode(name):
+    return "fused" if name in ("cfg4", "cfg4u", "cfg5") else "steps"
+
+
+def build_workloads(name, modes, scale, device):
+    """{mode: (step, info)} of one configuration, on shared inputs."""
     def sc(x, q=1024):
         return max(q, int(x * scale) // q * q)
+    modes = [m or default_mode(name) for m in modes]
     if name == "cfg1":
-        return make_ring_rs(4, sc(16 * MiB), "f32", mode, device)
+        return make_ring_rs(4, sc(16 * MiB), "f32", modes, device)
     if name == "cfg2":
-        return make_ring_rs(8, sc(256 * MiB), "bf16", mode, device, std=1e-2)
+        return make_ring_rs(8, sc(256 * MiB), "bf16", modes, device, std=1e-2)
     if name == "cfg3":
-        return make_rh_pair(sc(256 * MiB), device)
+        pair = make_rh_pair(sc(256 * MiB), device)
+        return {m: pair["steps"] for m in modes}
     if name == "cfg3full":
-        return make_rh_full(64, sc(512 * MiB, 1 << 16), mode, device)
+        return make_rh_full(64, sc(512 * MiB, 1 << 16), modes, device)
     if name == "cfg4":
-        return make_all_gather(16, sc(128 * MiB), mode, device)
+        return make_all_gather(16, sc(128 * MiB), modes, device)
     if name == "cfg4u":
-        return make_all_gather(16, sc(128 * MiB), mode, device, uneven=True)
+        return make_all_gather(16, sc(128 * MiB), modes, device, uneven=True)
     if name == "cfg5":
-        return make_kway(32, sc(32 * MiB), mode, device)
+        return make_kway(32, sc(32 * MiB), modes, device)
     raise ValueError(name)
 
 
+def build_workload(name, mode, scale, device):
+    mode = mode or default_mode(name)
+    return build_workloads(name, [mode], scale, device)[mode]
+
+
+# ---------------------------------------------------------------------------
+# timing
+# ---------------------------------------------------------------------------
+
+def time_steps(step, steps, warmup, lib):
+    """Warm-up calls, then `steps` timed calls between two events on the stream
+    the library launches on.  Returns device ms, wall ms and launches per step."""
+    import torch
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    launches0 = lib.launch_count()
+    start.record(stream)
+    for _ in range(steps):
+        step()
+    end.record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return start.elapsed_time(end), wall_ms, (lib.launch_count() - launches0) / steps
+
+
+def roofline_of(info, dev_ms, steps, launched):
+    """Roofline of the dominant kernel from the live timing: the timed region
+    holds nothing but that kernel's launches (plus, in faithful mode, copies),
+    so its mean launch time is region / launches and the bytes of a mean launch
+    are the step's kernel bytes / launches."""
+    if not (info["launches"] == info["kernel_launches"] or info["kernel_bytes"] == info["alg_bytes"]):
+        return None
+    step_kernel_bytes = (info["kernel_bytes"] * info["kernel_launches"]
+                         if info["launches"] == info["kernel_launches"] else info["kernel_bytes"])
+    kernel_ms = dev_ms / (steps * launched)
+    launch_bytes = step_kernel_bytes / launched
+    achieved = launch_bytes / (kernel_ms * 1e-3) / 1e9
+    return {"bound": "hbm", "kernel": info["kernel"], "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+            "bytes_per_launch": int(round(launch_bytes)), "avg_launch_ms": round(kernel_ms, 5)}
+
+
+def source_hash():
+    """Digest of the kernel sources: a counter reading taken from another
+    version of the kernels says nothing about this one."""
+    h = hashlib.sha256()
+    for f in ("pccl_kernels.h", "pccl_hip.hip"):
+        with open(os.path.join(ROOT, "sc2025-pccl-reproducer_amd", "csrc", f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def profiled_traffic(workload, mode, kernel, lib, scale):
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 counter runs
+    (profiles/traffic.json), or None with the reason: the entry must have been
+    taken with these kernel sources, the default tuning and the full size."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        table = json.load(open(path))
+    except Exception:                                         # noqa: BLE001
+        return None, "no profiles/traffic.json"
+    entry = table.get("entries", {}).get(f"{workload}:{mode}:{kernel}")
+    if entry is None:
+        return None, "no counter run recorded for this workload and mode"
+    if table.get("source_sha256_16") != source_hash():
+        return None, "recorded with other kernel sources than the ones loaded"
+    if scale != 1.0 or any(lib.get_tuning(k) != v for k, v in table.get("tuning", {}).items()):
+        return None, "recorded at the default tuning and full size, not this run's"
+    return entry, None
+
+
+def run_row(name, mode, step, info, steps, warmup, lib, verify=True):
+    dev_ms, wall_ms, launched = time_steps(step, steps, warmup, lib)
+    ms = dev_ms / steps
+    gbps = info["alg_bytes"] / (ms * 1e-3) / 1e9
+    roof = roofline_of(info, dev_ms, steps, launched)
+    ok = bool(info["verify"]()) if verify else None
+    row = {"workload": name, "mode": mode, "kernel": info["kernel"], "ms": round(ms, 4), "GBps": round(gbps, 1),
+           "frac": round(gbps / HBM_PEAK_GBPS, 4), "launches": launched,
+           "bytes_per_launch": roof["bytes_per_launch"] if roof else None,
+           "avg_launch_ms": roof["avg_launch_ms"] if roof else None,
+           "algorithmic_bytes": info["alg_bytes"], "steps": steps, "warmup": warmup,
+           "verified": ok, "verified_by": info.get("verify_how") if verify else None}
+    return row, roof, dev_ms, wall_ms, launched
+
+
 def ceilings(steps, warmup, device):
-    """GB/s of pure read, pure write, copy and add streams over 1 GiB buffers."""
+    """GB/s of pure read, pure write, copy and add streams over 1 GiB buffers, and
+    of read:write mixes with no data flowing from the loads to the stores."""
     import torch
     from pccl import _native, kernels
     lib = _native.load()
@@ -406,7 +578,7 @@ def ceilings(steps, warmup, device):
         return round(nbytes / (s.elapsed_time(e) / steps * 1e-3) / 1e9, 1)
 
     st = kernels.stream_handle()
-    return {
+    res = {
         "read_only": gbps(lambda: lib.probe_stream(0, a.data_ptr(), n, st), n),
         "write_only": gbps(lambda: lib.probe_stream(1, c.data_ptr(), n, st), n),
         "copy": gbps(lambda: kernels.copy(c, a), 2 * n),
@@ -414,6 +586,38 @@ def ceilings(steps, warmup, device):
         "torch_copy_": gbps(lambda: c.copy_(a), 2 * n),
         "torch_add_f32": gbps(lambda: torch.add(fa, fb, out=fc), 3 * n),
     }
+    del a, b, c, fa, fb, fc
+    # read:write mixes, the best of the probe's shapes (all streams per workgroup or
+    # one stream per workgroup; 1, 2 or 4 vectors per thread), beside the library
+    # kernel of the same mix on the same buffers
+    mixes = {}
+    for nr, nw, mib in ((2, 1, 1024), (8, 1, 256), (32, 1, 128), (1, 16, 128)):
+        nb = mib * MiB
+        rd = [torch.empty(nb // 4, device=device).normal_() for _ in range(nr)]
+        wr = [torch.empty(nb // 4, device=device) for _ in range(nw)]
+        rp, wp = [t.data_ptr() for t in rd], [t.data_ptr() for t in wr]
+        best, shape = 0.0, None
+        for sh in (0, 1):
+            for u in (1, 2, 4):
+                v = gbps(lambda: lib.probe_mix(rp, wp, nb, sh, u, st), (nr + nw) * nb)
+                if v > best:
+                    best, shape = v, f"shape {sh}, {u} vectors per thread"
+        if nw == 1 and nr == 2:
+            mine, kname = gbps(lambda: kernels.add(wr[0], rd[0], rd[1]), 3 * nb), "k_add_segs"
+        elif nw == 1:
+            mine, kname = gbps(lambda: kernels.reduce_kway(wr[0], rd, "ring", 1), (nr + 1) * nb), "k_reduce_kway"
+        else:
+            # nw shards of nb / nw bytes into nw outputs of nb bytes: nb read, nw * nb written
+            g_out = [w.view(torch.uint8) for w in wr]
+            g_in = [rd[0].view(torch.uint8)[q * (nb // nw):(q + 1) * (nb // nw)] for q in range(nw)]
+            mine, kname = gbps(lambda: kernels.all_gather_ranks(g_out, g_in, "ring", "fused"), (1 + nw) * nb), \
+                "k_gather_strips"
+            del g_out, g_in
+        mixes[f"{nr}r{nw}w_{mib}MiB"] = {"probe": best, "probe_shape": shape, "library_kernel": kname,
+                                         "library": mine, "library_over_probe": round(mine / best, 3)}
+        del rd, wr
+    res["mixes"] = mixes
+    return res
 
 
 def size_sweep(steps, warmup, device):
@@ -454,7 +658,8 @@ def size_sweep(steps, warmup, device):
 
 
 def latency_sweep(steps, warmup, device):
-    """Microseconds per call for launch-bound message sizes (bf16)."""
+    """Microseconds per call for launch-bound message sizes (bf16), through the
+    ordinary Python API unless a column says otherwise."""
     import torch
     from pccl import kernels
 
@@ -479,6 +684,7 @@ def latency_sweep(steps, warmup, device):
         B = max(8, n // P)
         ins = [_randn_bf16(P * B, 1.0, 10 + r, device) for r in range(P)]
         outs = [torch.empty(B, dtype=torch.bfloat16, device=device) for _ in range(P)]
+        gouts = [torch.empty(P * B, dtype=torch.bfloat16, device=device) for _ in range(P)]
         work = [torch.empty_like(t) for t in ins]
         graph = torch.cuda.CUDAGraph()             # the 7 step launches captured once
         kernels.reduce_scatter_ranks(outs, ins, "ring", "steps", work)
@@ -486,18 +692,79 @@ def latency_sweep(steps, warmup, device):
         with torch.cuda.graph(graph):
             kernels.reduce_scatter_ranks(outs, ins, "ring", "steps", work)
         plan_fused = kernels.plan_reduce_scatter(outs, ins, "ring", "fused")
-        plan_steps = kernels.plan_reduce_scatter(outs, ins, "ring", "steps", work)
         rows.append({
             "bytes": nbytes,
             "accumulate_us": round(us(lambda: kernels.accumulate(x, y)), 2),
             "copy_us": round(us(lambda: kernels.copy(z, x)), 2),
+            "ring_rs_p8_fused_us": round(us(lambda: kernels.reduce_scatter_ranks(outs, ins, "ring", "fused")), 2),
+            "ring_rs_p8_fused_plan_us": round(us(plan_fused), 2),
             "ring_rs_p8_steps_us": round(us(lambda: kernels.reduce_scatter_ranks(outs, ins, "ring", "steps", work)), 2),
             "ring_rs_p8_steps_graph_us": round(us(graph.replay), 2),
-            "ring_rs_p8_steps_plan_us": round(us(plan_steps), 2),
-            "ring_rs_p8_fused_plan_us": round(us(plan_fused), 2),
-            "ring_rs_p8_fused_us": round(us(lambda: kernels.reduce_scatter_ranks(outs, ins, "ring", "fused")), 2),
+            "all_gather_p8_fused_us": round(us(lambda: kernels.all_gather_ranks(gouts, outs, "ring", "fused")), 2),
         })
     return rows
+
+
+def drop_in(device, steps=5, warmup=2):
+    """Wall time of the reference-shaped per-rank calls at the cfg2 size: 8
+    virtual ranks (one Python thread each, as `mpirun -np 8` would start them)
+    call pccl._reduce_scatter / pccl.reduce_scatter_2D / pccl.all_gather_2D with
+    use_pccl_cpp_backend=True (pccl/reduce_scatter.py:164-235, pccl/all_gather.py:136-159)."""
+    import torch
+    import pccl
+    P, total = 8, 256 * MiB
+    B = total // P
+    ins = [_randn_bf16(total, 1e-2, 50 + r, device) for r in range(P)]
+    outs = [torch.empty(B, dtype=torch.bfloat16, device=device) for _ in range(P)]
+    gouts = [torch.empty(total, dtype=torch.bfloat16, device=device) for _ in range(P)]
+    world = pccl.VirtualWorld(P, device)
+    res = {}
+
+    def timed(name, call, setup=None):
+        def rank_main(comm):
+            r = comm.Get_rank()
+            ctx = setup(comm) if setup else None
+            t0 = None
+            for it in range(warmup + steps):
+                if it == warmup:
+                    comm.Barrier()
+                    if r == 0:
+                        torch.cuda.synchronize()
+                    comm.Barrier()
+                    t0 = time.perf_counter()
+                call(comm, r, ctx)
+            comm.Barrier()
+            if r == 0:
+                torch.cuda.synchronize()
+                return (time.perf_counter() - t0) * 1e3 / steps
+            return None
+        res[name] = round(world.run(rank_main)[0], 4)
+
+    def grid(comm):
+        return pccl.ProcessGroups(4, 2, inner_group_backend="mpi", outer_group_backend="mpi", comm=comm)
+
+    timed("_reduce_scatter_ring_ms",
+          lambda comm, r, _: pccl._reduce_scatter(outs[r], ins[r], group=comm, use_pccl_cpp_backend=True))
+    timed("reduce_scatter_2D_4x2_ring_ms",
+          lambda comm, r, pg: pccl.reduce_scatter_2D(outs[r], ins[r], group=pg, use_pccl_cpp_backend=True), grid)
+    timed("reduce_scatter_2D_4x2_halving_ms",
+          lambda comm, r, pg: pccl.reduce_scatter_2D(outs[r], ins[r], group=pg, use_rh=True,
+                                                     use_pccl_cpp_backend=True), grid)
+    timed("all_gather_2D_4x2_doubling_ms",
+          lambda comm, r, pg: pccl.all_gather_2D(gouts[r], outs[r], group=pg, use_rd=True,
+                                                 use_pccl_cpp_backend=True), grid)
+    # the same collective through the single-thread driver call, for scale
+    from pccl import kernels
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        kernels.reduce_scatter_ranks(outs, ins, "ring")
+    torch.cuda.synchronize()
+    res["driver_reduce_scatter_ranks_ring_ms"] = round((time.perf_counter() - t0) * 1e3 / steps, 4)
+    res["what"] = (f"wall ms per call, {P} virtual ranks = {P} Python threads meeting per call, bf16, "
+                   f"{total * 2 // MiB} MiB per rank, default execution mode ({kernels.DEFAULT_MODE}), "
+                   f"{warmup} warm-up + {steps} timed calls")
+    return res
 
 
 # ---------------------------------------------------------------------------
@@ -574,6 +841,11 @@ def cpu_baseline(info):
 
 # ---------------------------------------------------------------------------
 
+TUNING_KEYS = ("grid_cap", "unroll", "unroll_copy", "nt_load", "nt_store", "launch_mib", "gather_strip",
+               "gather_split", "unroll_gather", "gather_nt", "lds_pad", "lds_pad_copy", "lds_pad_kway",
+               "lds_pad_gather")
+
+
 def main():
     global LAYOUT
     args = parse_args()
@@ -601,8 +873,9 @@ def main():
             "metric": METRIC, "value": res["add_2r1w_f32"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": round(3 * (1 << 30) / res["add_2r1w_f32"] / 1e6, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-            "config": {"workload": "ceilings: plain streams over 1 GiB buffers; value = the library's add kernel",
-                       "GBps": res}, "roofline": None, "cpu_baseline": None}), flush=True)
+            "config": {"workload": "ceilings: plain streams over 1 GiB buffers and read:write mixes; "
+                                   "value = the library's add kernel", "GBps": res},
+            "roofline": None, "cpu_baseline": None}), flush=True)
         return 0
 
     if args.workload == "sweep":
@@ -632,26 +905,18 @@ def main():
                        "latency_us": rows}, "roofline": None, "cpu_baseline": None}), flush=True)
         return 0
 
-    step, info = build_workload(args.workload, args.mode, args.scale, device)
+    everything = args.workload == "all"
+    head_name = "cfg2" if everything else args.workload
+    head_mode = (args.mode or default_mode(head_name)) if not everything else "steps"
+    want_modes = [head_mode]
+    if everything:
+        want_modes += [m for n, m in ALL_ROWS if n == head_name and m != head_mode]
+    built = build_workloads(head_name, want_modes, args.scale, device)
+    step, info = built[head_mode]
     torch.cuda.synchronize()
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    stream = torch.cuda.current_stream()           # the stream the library launches on
-    start = torch.cuda.Event(enable_timing=True)
-    end = torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    launches0 = lib.launch_count()
-    start.record(stream)
-    for _ in range(args.steps):
-        step()
-    end.record(stream)
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    dev_ms = start.elapsed_time(end)
-    # a step of a schedule goes out as several launches of bounded size (launch_mib)
-    launched = (lib.launch_count() - launches0) / args.steps
+    row, roof, dev_ms, wall_ms, launched = run_row(head_name, head_mode, step, info, args.steps, args.warmup, lib,
+                                                   verify=False)
     ms_per_step = dev_ms / args.steps
     value = info["alg_bytes"] / (ms_per_step * 1e-3) / 1e9
 
@@ -666,32 +931,46 @@ def main():
 
     ok = None
     if not args.no_verify:
+        step()                            # the outputs of this mode, not of a later one
         ok = bool(info["verify"]())
+    if roof:
+        roof["traffic"], roof["traffic_note"] = profiled_traffic(head_name, head_mode, info["kernel"], lib, args.scale)
+        if roof["traffic"] is not None:
+            roof["traffic_note"] = ("HBM bytes per launch from the rocprofv3 FETCH_SIZE/WRITE_SIZE runs summarised in "
+                                    "profiles/ (same kernel sources, default tuning, full size); not measured in this run")
 
-    # the timed region holds nothing but the dominant kernel's launches (plus, in
-    # faithful mode, the copies), so its mean launch time is region / launches and
-    # the bytes of a mean launch are the step's kernel bytes / launches
-    if info["launches"] == info["kernel_launches"] or info["kernel_bytes"] == info["alg_bytes"]:
-        step_kernel_bytes = (info["kernel_bytes"] * info["kernel_launches"]
-                             if info["launches"] == info["kernel_launches"] else info["kernel_bytes"])
-        kernel_ms = dev_ms / (args.steps * launched)
-        launch_bytes = step_kernel_bytes / launched
-    else:
-        kernel_ms = None
-    roof = None
-    if kernel_ms:
-        achieved = launch_bytes / (kernel_ms * 1e-3) / 1e9
-        traffic = None
-        tfile = os.path.join(ROOT, "profiles", "traffic.json")
-        if os.path.exists(tfile):
-            try:
-                traffic = json.load(open(tfile)).get(f"{args.workload}:{info['kernel']}")
-            except Exception:                                 # noqa: BLE001
-                traffic = None
-        roof = {"bound": "hbm", "kernel": info["kernel"], "achieved": round(achieved, 1),
-                "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                "traffic": traffic, "bytes_per_launch": int(round(launch_bytes)),
-                "avg_launch_ms": round(kernel_ms, 5)}
+    rows, all_ok = [], ok in (None, True)
+    extra = {}
+    if everything:
+        sub_steps, sub_warm = min(args.steps, 10), min(args.warmup, 3)
+
+        def add_row(name, mode, step_fn, info_):
+            nonlocal all_ok
+            r, _, _, _, _ = run_row(name, mode, step_fn, info_, sub_steps, sub_warm, lib, verify=not args.no_verify)
+            rows.append(r)
+            all_ok = all_ok and r["verified"] in (None, True)
+
+        for m in want_modes[1:]:
+            add_row(head_name, m, *built[m])
+        del built, step
+        info = {k: v for k, v in info.items() if k != "verify"}
+        torch.cuda.empty_cache()
+        todo = {}
+        for n, m in ALL_ROWS:
+            if n != head_name:
+                todo.setdefault(n, []).append(m)
+        for n, modes in todo.items():
+            group = build_workloads(n, modes, args.scale, device)
+            for m in modes:
+                add_row(n, m, *group[m])
+            del group
+            torch.cuda.empty_cache()
+        rows.sort(key=lambda r: [x for x, _ in ALL_ROWS].index(r["workload"]))
+        extra["latency_us"] = latency_sweep(50, 10, device)
+        extra["ceilings"] = ceilings(10, 3, device)
+        torch.cuda.empty_cache()
+        extra["drop_in"] = drop_in(device)
+        torch.cuda.empty_cache()
 
     cpu = None if args.no_cpu_baseline else cpu_baseline(info)
 
@@ -699,14 +978,18 @@ def main():
         "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": info["dtype"], "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {info['desc']}", "algorithmic_bytes_per_step": info["alg_bytes"],
+        "config": {"workload": f"{head_name}: {info['desc']}", "algorithmic_bytes_per_step": info["alg_bytes"],
                    "launches_per_step": launched, "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
-                   "wall_ms_per_step": round(wall_ms / args.steps, 4), "verified": ok, "layout": LAYOUT,
-                   "tuning": {k: lib.get_tuning(k) for k in ("grid_cap", "unroll", "unroll_copy", "nt_load", "nt_store", "launch_mib")}},
+                   "wall_ms_per_step": round(wall_ms / args.steps, 4), "verified": ok,
+                   "verified_by": info.get("verify_how"), "layout": LAYOUT,
+                   "tuning": {k: lib.get_tuning(k) for k in TUNING_KEYS}},
         "roofline": roof, "cpu_baseline": cpu,
     }
+    if everything:
+        out["config"]["workloads"] = rows
+        out["config"].update(extra)
     print(json.dumps(out), flush=True)
-    return 0 if ok in (None, True) else 1
+    return 0 if all_ok else 1
 
 
 if __name__ == "__main__":

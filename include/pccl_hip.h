@@ -46,13 +46,13 @@ extern "C" {
 #define PCCL_HIP_ABI_VERSION 1
 
 /* Largest number of segments / shards one LAUNCH takes (their pointers travel
- * in the kernel arguments): the limit of the batched kernels, of every fused
- * mode and of the 2-D entry points. */
+ * in the kernel arguments): the limit of the batched kernels, of the uneven
+ * all_gather and of the 2-D entry points. */
 #define PCCL_HIP_MAX_RANKS 64
 
-/* Largest number of virtual ranks of the per-step (and faithful) modes of
- * pccl_hip_reduce_scatter_virtual / pccl_hip_all_gather_virtual: a step over
- * more than PCCL_HIP_MAX_RANKS ranks goes out as several launches. */
+/* Largest number of virtual ranks of pccl_hip_reduce_scatter_virtual /
+ * pccl_hip_all_gather_virtual: a step (or a fused collective) over more than
+ * PCCL_HIP_MAX_RANKS ranks goes out as several launches. */
 #define PCCL_HIP_MAX_VIRTUAL_RANKS 4096
 
 /* Element types.  bf16 sums are computed as RNE_bf16(float(a) + float(b)) at
@@ -186,12 +186,17 @@ int pccl_hip_block_transpose(void* dst, const void* src, size_t rows,
  *   inputs[r]  : rank r's input, P*B elements (read only)
  *   outputs[r] : rank r's output, B elements = sum_k inputs[k][r*B:(r+1)*B]
  *   work[r]    : rank r's workspace, P*B elements; may be NULL as a whole
- *                for PCCL_HIP_MODE_FUSED and for P <= 2
+ *                for P <= 2 and for PCCL_HIP_MODE_FUSED (except "recursive"
+ *                with P > PCCL_HIP_MAX_RANKS, see below)
  *   algorithm  : "ring" or "recursive" (recursive needs P a power of two);
  *                any other string is an error, as at pccl.cpp:83.
  * The summation order of each output block is that of the named algorithm in
- * every mode.  1 <= P <= PCCL_HIP_MAX_VIRTUAL_RANKS (PCCL_HIP_MAX_RANKS for
- * PCCL_HIP_MODE_FUSED). */
+ * every mode.  1 <= P <= PCCL_HIP_MAX_VIRTUAL_RANKS.  PCCL_HIP_MODE_FUSED is
+ * one launch up to PCCL_HIP_MAX_RANKS ranks.  Beyond, "ring" folds every
+ * output block in ceil((P-1)/63) launches of at most 64 operands, the running
+ * sum (kept in the output) being the first operand of the next launch, and
+ * "recursive" runs halving rounds step by step until groups of 64 ranks
+ * remain (this needs work[]) and finishes each group with one launch. */
 int pccl_hip_reduce_scatter_virtual(void* const* outputs,
                                     const void* const* inputs,
                                     void* const* work, int P, size_t B,
@@ -235,8 +240,8 @@ int pccl_hip_reduce_scatter_virtual_noalloc(void* const* outputs,
  *                (the ring schedule the reference leaves to MPI_Allgather,
  *                pccl/all_gather.py:124-128).
  * PCCL_HIP_MODE_STEPS replays one batched copy per step;
- * PCCL_HIP_MODE_FUSED places every shard directly; FAITHFUL == STEPS.
- * P limits as for pccl_hip_reduce_scatter_virtual. */
+ * PCCL_HIP_MODE_FUSED places every shard directly (one launch per 64 shards
+ * and 64 outputs); FAITHFUL == STEPS.  1 <= P <= PCCL_HIP_MAX_VIRTUAL_RANKS. */
 int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs,
                                 int P, size_t block_bytes,
                                 const char* algorithm, int mode, void* stream);
@@ -293,6 +298,19 @@ int pccl_hip_all_gather_2d_virtual(void* const* outputs,
  * ceiling the 2-reads-1-write kernels are judged against.  No counterpart in
  * the reference.  buf must be 16-byte aligned, nbytes >= 4096. */
 int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream);
+
+/* A read:write MIX in one launch: nr read streams and nw write streams of
+ * nbytes bytes each, with no data flowing from the loads to the stores (the
+ * loads are folded and dropped, the stores write a constant).  Timing it gives
+ * what the device sustains for the 2:1 mix of the add kernels, the k:1 mix of
+ * the fused reduce or the 1:P mix of the all_gather placement when nothing but
+ * the memory system is in the way.  shape 0: workgroup t serves tile t of every
+ * stream; shape 1: every workgroup serves one stream.  vectors = 128-bit
+ * vectors per thread and stream (1, 2 or 4).  No counterpart in the reference.
+ * Streams must be 16-byte aligned, nbytes a multiple of 16, nr, nw <= 64. */
+int pccl_hip_probe_mix(const void* const* reads, int nr, void* const* writes,
+                       int nw, size_t nbytes, int shape, int vectors,
+                       void* stream);
 
 /* ---- launch tuning (for measurement) ------------------------------------
  * key: "grid_cap" (max workgroups per launch, 0 = one tile per workgroup),

@@ -719,25 +719,27 @@ int pccl_hip_block_transpose(void* dst, const void* src, size_t rows, size_t col
   return launch_status(what);
 }
 
-int pccl_hip_all_gather_uneven_virtual(void* const* outputs, const void* const* inputs,
-                                       const size_t* nbytes, const size_t* dst_off, int P,
-                                       void* stream) {
-  const char* what = "pccl_hip_all_gather_uneven_virtual";
-  if (P < 1 || P > kMaxSeg) return fail(PCCL_HIP_EINVAL, "%s: P = %d outside [1, %d]", what, P, kMaxSeg);
-  if (!nbytes || !dst_off) return fail(PCCL_HIP_EINVAL, "%s: NULL size table", what);
-  if (int rc = check_table((const void* const*)outputs, P, what, "outputs")) return rc;
-  if (!inputs) return fail(PCCL_HIP_EINVAL, "%s: inputs is NULL", what);
+}  // extern "C"
+
+namespace {
+
+// Places `nshards` shards (shard k: nbytes[k] bytes at byte offset dst_off[k]) into
+// each of `nout` outputs in one launch; both counts at most kMaxSeg.
+int gather_place_all(void* const* outputs, int nout, const void* const* inputs, const size_t* nbytes,
+                     const size_t* dst_off, int nshards, void* stream, const char* what) {
+  const int P = nshards;
   GatherArgs args;
   size_t longest = 0, payload = 0;
+  for (int r = 0; r < nout; ++r) args.outs[r] = outputs[r];
   for (int k = 0; k < P; ++k) {
     if (nbytes[k] && !inputs[k]) return fail(PCCL_HIP_EINVAL, "%s: inputs[%d] is NULL", what, k);
-    args.outs[k] = outputs[k]; args.ins[k] = inputs[k];
+    args.ins[k] = inputs[k];
     args.nbytes[k] = nbytes[k]; args.dst_off[k] = dst_off[k];
     longest = nbytes[k] > longest ? nbytes[k] : longest;
     payload += nbytes[k];
   }
   if (longest == 0) return PCCL_HIP_OK;
-  const size_t moved = ((size_t)P + 1) * payload;   // every shard read, and written to P outputs
+  const size_t moved = ((size_t)nout + 1) * payload;   // every shard read, and written to nout outputs
   Tune t = current_tune(false, moved);
   // Two kernels.  Time-blocked strips (k_gather_strips): an XCD walks a strip of
   // its tiles once per output, so it feeds one write stream at a time and re-reads
@@ -754,7 +756,7 @@ int pccl_hip_all_gather_uneven_virtual(void* const* outputs, const void* const* 
   if (strip < 0) {
     long from = g_gather_strip_from.load(std::memory_order_relaxed);
     if (from < 0) from = kStripFrom;
-    strip = (P >= 2 && longest >= (size_t)from) ? kStripItems : 0;
+    strip = (nout >= 2 && longest >= (size_t)from) ? kStripItems : 0;
   }
   const long unroll_set = g_unroll_gather.load(std::memory_order_relaxed);
   const long pad_set = g_lds_pad_gather.load(std::memory_order_relaxed);
@@ -767,15 +769,15 @@ int pccl_hip_all_gather_uneven_virtual(void* const* outputs, const void* const* 
     if (g_gather_strip.load(std::memory_order_relaxed) < 0 && items + items / 4 + 1 < (size_t)strip)
       strip = (long)(items + items / 4 + 1);
     const size_t n_local = (items + (size_t)strip - 1) / (size_t)strip * (size_t)strip;
-    if (int rc = check_work_items((size_t)P * (size_t)P * kXcds, n_local, what)) return rc;
+    if (int rc = check_work_items((size_t)P * (size_t)nout * kXcds, n_local, what)) return rc;
     const bool nts = stream_hint(g_gather_nt.load(), moved);
     hipStream_t st = (hipStream_t)stream;
 #define PCCL_STRIPS(UV)                                                                                              \
   case UV:                                                                                                          \
-    if (nts) hipLaunchKernelGGL((k_gather_strips<UV, false, true>), dim3(grid), dim3(kThreads), lds, st, args, P, P, (uint32_t)n_local, (uint32_t)strip, span); \
-    else hipLaunchKernelGGL((k_gather_strips<UV, false, false>), dim3(grid), dim3(kThreads), lds, st, args, P, P, (uint32_t)n_local, (uint32_t)strip, span);    \
+    if (nts) hipLaunchKernelGGL((k_gather_strips<UV, false, true>), dim3(grid), dim3(kThreads), lds, st, args, P, nout, (uint32_t)n_local, (uint32_t)strip, span); \
+    else hipLaunchKernelGGL((k_gather_strips<UV, false, false>), dim3(grid), dim3(kThreads), lds, st, args, P, nout, (uint32_t)n_local, (uint32_t)strip, span);    \
     break;
-    for_spans((size_t)P * (size_t)P * kXcds * n_local, 0, 1, 0, [&](Span span, unsigned grid) {
+    for_spans((size_t)P * (size_t)nout * kXcds * n_local, 0, 1, 0, [&](Span span, unsigned grid) {
       switch (U) {
         PCCL_STRIPS(1)
         PCCL_STRIPS(2)
@@ -794,13 +796,28 @@ int pccl_hip_all_gather_uneven_virtual(void* const* outputs, const void* const* 
   // (P = 32), +15 % (P = 64); more than four streams per workgroup or more
   // workgroups per tile are both slower.
   int split = (int)g_gather_split.load(std::memory_order_relaxed);
-  if (split <= 0) split = (P + 3) / 4;
-  if (split > P) split = P;
-  GatherLaunch l{&args, P, P, split, copy_tiles_for(longest, t.unroll), stream_hint(g_gather_nt.load(), moved),
+  if (split <= 0) split = (nout + 3) / 4;
+  if (split > nout) split = nout;
+  GatherLaunch l{&args, P, nout, split, copy_tiles_for(longest, t.unroll), stream_hint(g_gather_nt.load(), moved),
                  lds, (hipStream_t)stream};
   if (int rc = check_work_items((size_t)P * (size_t)split, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);
+}
+
+}  // namespace
+
+extern "C" {
+
+int pccl_hip_all_gather_uneven_virtual(void* const* outputs, const void* const* inputs,
+                                       const size_t* nbytes, const size_t* dst_off, int P,
+                                       void* stream) {
+  const char* what = "pccl_hip_all_gather_uneven_virtual";
+  if (P < 1 || P > kMaxSeg) return fail(PCCL_HIP_EINVAL, "%s: P = %d outside [1, %d]", what, P, kMaxSeg);
+  if (!nbytes || !dst_off) return fail(PCCL_HIP_EINVAL, "%s: NULL size table", what);
+  if (int rc = check_table((const void* const*)outputs, P, what, "outputs")) return rc;
+  if (!inputs) return fail(PCCL_HIP_EINVAL, "%s: inputs is NULL", what);
+  return gather_place_all(outputs, P, inputs, nbytes, dst_off, P, stream, what);
 }
 
 }  // extern "C"
@@ -833,10 +850,10 @@ int reduce_scatter_ranks(void* const* outputs, const void* const* inputs, void* 
                          const char* what) {
   if (int rc = check_reduce_scatter_args(outputs, inputs, P, dtype, algorithm, mode, what)) return rc;
   const bool ring = !strcmp(algorithm, "ring");
-  if (mode == PCCL_HIP_MODE_FUSED && P > kMaxSeg)
-    return fail(PCCL_HIP_EINVAL, "%s: the fused mode folds at most %d ranks in one launch, got P = %d", what,
-                kMaxSeg, P);
-  const bool need_work = (mode == PCCL_HIP_MODE_FAITHFUL && P > 1) || (mode == PCCL_HIP_MODE_STEPS && P > 2);
+  // beyond the shards of one launch the fused halving order runs its first rounds step by step (see below)
+  const bool fused_rounds = mode == PCCL_HIP_MODE_FUSED && !ring && P > kMaxSeg;
+  const bool need_work = (mode == PCCL_HIP_MODE_FAITHFUL && P > 1) || (mode == PCCL_HIP_MODE_STEPS && P > 2) ||
+                         fused_rounds;
   if (need_work) if (int rc = check_table((const void* const*)work, P, what, "work")) return rc;
   if (B == 0) return PCCL_HIP_OK;
   hipStream_t st = (hipStream_t)stream;
@@ -850,12 +867,40 @@ int reduce_scatter_ranks(void* const* outputs, const void* const* inputs, void* 
     return launch_copy(c, 1, st, what);
   }
 
-  if (mode == PCCL_HIP_MODE_FUSED) {
+  if (mode == PCCL_HIP_MODE_FUSED && P <= kMaxSeg) {
     KwayArgs args;
     for (int r = 0; r < P; ++r) { args.shard[r] = inputs[r]; args.out[r] = outputs[r]; args.eoff[r] = (size_t)r * B; }
     // ring: block j is folded from rank j+1 on; halving: the butterfly rooted at rank j
     return launch_kway(args, P, P, P, B, dtype, ring ? PCCL_HIP_ORDER_RING : PCCL_HIP_ORDER_HALVING,
                        ring ? 1 : 0, 1, st, what);
+  }
+
+  if (mode == PCCL_HIP_MODE_FUSED && ring) {
+    // More ranks than one launch has shard pointers: the left fold of block j is cut
+    // into launches of at most kMaxSeg operands, and every launch after the first
+    // takes the running sum (already in output j) as its first operand.  A partial
+    // sum is stored in the element type, which is what every hop rounds to anyway,
+    // so the bits are those of the single fold.  One chain of launches per output.
+    for (int j = 0; j < P; ++j) {
+      int rank = (j + 1) % P;   // the fold of block j starts at rank j+1 and ends with rank j
+      int left = P;
+      bool running = false;
+      while (left > 0) {
+        KwayArgs args;
+        int k = 0;
+        if (running) args.shard[k++] = outputs[j];
+        while (k < kMaxSeg && left > 0) {
+          args.shard[k++] = (const uint8_t*)inputs[rank] + (size_t)j * B * es;
+          rank = rank + 1 == P ? 0 : rank + 1;
+          --left;
+        }
+        args.out[0] = outputs[j];
+        args.eoff[0] = 0;
+        if (int rc = launch_kway(args, k, k, 1, B, dtype, PCCL_HIP_ORDER_RING, 0, 1, st, what)) return rc;
+        running = true;
+      }
+    }
+    return PCCL_HIP_OK;
   }
 
   const bool faithful = mode == PCCL_HIP_MODE_FAITHFUL;
@@ -899,6 +944,19 @@ int reduce_scatter_ranks(void* const* outputs, const void* const* inputs, void* 
   int rounds = 0;
   while ((1 << rounds) < P) ++rounds;
   for (int round = 0; round < rounds; ++round) {
+    if (fused_rounds && (P >> round) == kMaxSeg) {
+      // The rest of the butterfly stays inside groups of kMaxSeg ranks whose partial
+      // sums lie in the work buffers: one fused launch per group finishes it.
+      for (int g0 = 0; g0 < P; g0 += kMaxSeg) {
+        KwayArgs args;
+        for (int q = 0; q < kMaxSeg; ++q) {
+          args.shard[q] = work[g0 + q]; args.out[q] = outputs[g0 + q]; args.eoff[q] = (size_t)(g0 + q) * B;
+        }
+        if (int rc = launch_kway(args, kMaxSeg, kMaxSeg, kMaxSeg, B, dtype, PCCL_HIP_ORDER_HALVING, 0, 1, st, what))
+          return rc;
+      }
+      return PCCL_HIP_OK;
+    }
     const bool from_inputs = !faithful && round == 0;
     const bool to_outputs = !faithful && round == rounds - 1;
     if (P <= kMaxSeg) {   // the pairwise kernel finds partner and halves from (rank, round) itself
@@ -1004,9 +1062,6 @@ int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs,
     return fail(PCCL_HIP_EINVAL, "%s: recursive doubling needs a power-of-two P, got %d", what, P);
   if (mode != PCCL_HIP_MODE_STEPS && mode != PCCL_HIP_MODE_FUSED && mode != PCCL_HIP_MODE_FAITHFUL)
     return fail(PCCL_HIP_EINVAL, "%s: unknown mode %d", what, mode);
-  if (mode == PCCL_HIP_MODE_FUSED && P > kMaxSeg)
-    return fail(PCCL_HIP_EINVAL, "%s: the fused mode places at most %d shards in one launch, got P = %d", what,
-                kMaxSeg, P);
   if (int rc = check_table((const void* const*)outputs, P, what, "outputs")) return rc;
   if (int rc = check_table(inputs, P, what, "inputs")) return rc;
   if (block_bytes == 0) return PCCL_HIP_OK;
@@ -1014,9 +1069,17 @@ int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs,
   CallBytes footprint(((size_t)P * P + P) * block_bytes);   // P shards and P outputs of P blocks
 
   if (mode == PCCL_HIP_MODE_FUSED) {
+    // one launch places up to kMaxSeg shards into up to kMaxSeg outputs
     size_t nbytes[kMaxSeg], off[kMaxSeg];
-    for (int k = 0; k < P; ++k) { nbytes[k] = block_bytes; off[k] = (size_t)k * block_bytes; }
-    return pccl_hip_all_gather_uneven_virtual(outputs, inputs, nbytes, off, P, stream);
+    for (int k0 = 0; k0 < P; k0 += kMaxSeg) {
+      const int nk = P - k0 < kMaxSeg ? P - k0 : kMaxSeg;
+      for (int k = 0; k < nk; ++k) { nbytes[k] = block_bytes; off[k] = (size_t)(k0 + k) * block_bytes; }
+      for (int r0 = 0; r0 < P; r0 += kMaxSeg) {
+        const int nr = P - r0 < kMaxSeg ? P - r0 : kMaxSeg;
+        if (int rc = gather_place_all(outputs + r0, nr, inputs + k0, nbytes, off, nk, stream, what)) return rc;
+      }
+    }
+    return PCCL_HIP_OK;
   }
 
   // out[r][r] <- in[r]   (pccl/src/all_gather.cpp:31-35)
@@ -1340,6 +1403,35 @@ int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream) {
   else
     hipLaunchKernelGGL((k_probe_write<1, false>), dim3((unsigned)tiles), dim3(kThreads), 0, st, (u32x4*)buf, nvec,
                        0x3f803f80u);
+  g_launches.fetch_add(1, std::memory_order_relaxed);
+  return launch_status(what);
+}
+
+int pccl_hip_probe_mix(const void* const* reads, int nr, void* const* writes, int nw, size_t nbytes,
+                       int shape, int vectors, void* stream) {
+  const char* what = "pccl_hip_probe_mix";
+  if (nr < 0 || nw < 0 || nr > kMaxSeg || nw > kMaxSeg || nr + nw < 1)
+    return fail(PCCL_HIP_EINVAL, "%s: need 0 <= nr, nw <= %d and nr + nw >= 1", what, kMaxSeg);
+  if (shape != 0 && shape != 1) return fail(PCCL_HIP_EINVAL, "%s: shape must be 0 (one workgroup, all streams) or 1 (one stream per workgroup)", what);
+  if (vectors != 1 && vectors != 2 && vectors != 4) return fail(PCCL_HIP_EINVAL, "%s: vectors per thread must be 1, 2 or 4", what);
+  if (nbytes < 4096 || (nbytes & 15u)) return fail(PCCL_HIP_EINVAL, "%s: streams must hold a multiple of 16 and at least 4096 bytes", what);
+  if (nr) if (int rc = check_table(reads, nr, what, "reads")) return rc;
+  if (nw) if (int rc = check_table((const void* const*)writes, nw, what, "writes")) return rc;
+  MixArgs args;
+  for (int q = 0; q < nr; ++q) { if (!is16(reads[q])) return fail(PCCL_HIP_EINVAL, "%s: reads[%d] is not 16-byte aligned", what, q); args.rd[q] = reads[q]; }
+  for (int q = 0; q < nw; ++q) { if (!is16(writes[q])) return fail(PCCL_HIP_EINVAL, "%s: writes[%d] is not 16-byte aligned", what, q); args.wr[q] = writes[q]; }
+  const size_t nvec = nbytes / 16;
+  const size_t per_tile = (size_t)kThreads * (size_t)vectors;
+  size_t tiles = (nvec + per_tile - 1) / per_tile;
+  if (shape == 1) tiles *= (size_t)(nr + nw);
+  if (tiles > kMaxGrid) return fail(PCCL_HIP_EINVAL, "%s: streams too long for one launch", what);
+  hipStream_t st = (hipStream_t)stream;
+  const unsigned grid = (unsigned)tiles;
+  switch (vectors) {
+    case 1: hipLaunchKernelGGL((k_probe_mix<1, true, true>), dim3(grid), dim3(kThreads), 0, st, args, nr, nw, nvec, shape, 0x3f803f80u); break;
+    case 2: hipLaunchKernelGGL((k_probe_mix<2, true, true>), dim3(grid), dim3(kThreads), 0, st, args, nr, nw, nvec, shape, 0x3f803f80u); break;
+    default: hipLaunchKernelGGL((k_probe_mix<4, true, true>), dim3(grid), dim3(kThreads), 0, st, args, nr, nw, nvec, shape, 0x3f803f80u); break;
+  }
   g_launches.fetch_add(1, std::memory_order_relaxed);
   return launch_status(what);
 }

@@ -662,6 +662,68 @@ __global__ __launch_bounds__(kThreads) void k_probe_write(u32x4* dst, size_t nve
   }
 }
 
+struct MixArgs {
+  const void* rd[kMaxSeg];
+  void* wr[kMaxSeg];
+};
+
+// nr read streams and nw write streams of nvec vectors each in one launch, with
+// no data flowing from the loads to the stores: what the device sustains for a
+// given read:write mix when nothing but the memory system is in the way.
+//   shape 0: workgroup t loads tile t of every read stream and stores tile t of
+//            every write stream (the access shape of the add and fold kernels);
+//   shape 1: every workgroup serves ONE stream: workgroup w tile w / (nr + nw)
+//            of stream w % (nr + nw).
+// Loads are folded with xor and stored only on a value random data never hits.
+template <int U, bool NTL, bool NTS>
+__global__ __launch_bounds__(kThreads) void k_probe_mix(MixArgs t, int nr, int nw, size_t nvec, int shape,
+                                                       uint32_t value) {
+  const u32x4 v4 = {value, value, value, value};
+  u32x4 acc = {0, 0, 0, 0};
+  if (shape == 0) {
+    const size_t base = (size_t)blockIdx.x * (kThreads * U) + threadIdx.x;
+    for (int q = 0; q < nr; ++q) {
+      u32x4 x[U];
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const size_t v = base + (size_t)j * kThreads;
+        x[j] = v < nvec ? ld16<NTL>((const u32x4*)t.rd[q] + v) : u32x4{0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int j = 0; j < U; ++j) acc ^= x[j];
+    }
+    for (int q = 0; q < nw; ++q) {
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const size_t v = base + (size_t)j * kThreads;
+        if (v < nvec) st16<NTS>((u32x4*)t.wr[q] + v, v4);
+      }
+    }
+  } else {
+    const unsigned streams = (unsigned)(nr + nw);
+    const unsigned sidx = blockIdx.x % streams;
+    const size_t base = (size_t)(blockIdx.x / streams) * (kThreads * U) + threadIdx.x;
+    if (sidx < (unsigned)nr) {
+      u32x4 x[U];
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const size_t v = base + (size_t)j * kThreads;
+        x[j] = v < nvec ? ld16<NTL>((const u32x4*)t.rd[sidx] + v) : u32x4{0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int j = 0; j < U; ++j) acc ^= x[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const size_t v = base + (size_t)j * kThreads;
+        if (v < nvec) st16<NTS>((u32x4*)t.wr[sidx - nr] + v, v4);
+      }
+    }
+  }
+  if (nw > 0 && acc.x == 0x9e3779b9u && acc.y == 0x7f4a7c15u && acc.z == 0xf39cc060u && acc.w == 0x5cedc834u)
+    ((u32x4*)t.wr[0])[threadIdx.x] = acc;
+}
+
 struct KwayArgs {
   const void* shard[kMaxSeg];
   void* out[kMaxSeg];

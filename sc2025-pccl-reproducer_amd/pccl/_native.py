@@ -60,6 +60,7 @@ SIGNATURES = {
                                                   _int, _vp]),
     "pccl_hip_all_gather_2d_virtual": (_int, [_vpp, _vpp, _vpp, _int, _int, _sz, ctypes.c_char_p, _int, _vp]),
     "pccl_hip_probe_stream": (_int, [_int, _vp, _sz, _vp]),
+    "pccl_hip_probe_mix": (_int, [_vpp, _int, _vpp, _int, _sz, _int, _int, _vp]),
     "pccl_hip_set_tuning": (_int, [ctypes.c_char_p, ctypes.c_long]),
     "pccl_hip_get_tuning": (ctypes.c_long, [ctypes.c_char_p]),
     "pccl_hip_launch_count": (ctypes.c_ulonglong, []),
@@ -194,6 +195,12 @@ class NativeLib:
 
     def probe_stream(self, kind, buf, nbytes, stream=0):
         self._check(self._lib.pccl_hip_probe_stream(kind, buf, nbytes, stream))
+
+
+    def probe_mix(self, reads, writes, nbytes, shape=0, vectors=4, stream=0):
+        self._check(self._lib.pccl_hip_probe_mix(_ptr_table(reads) if reads else None, len(reads),
+                                                 _ptr_table(writes) if writes else None, len(writes), nbytes,
+                                                 shape, vectors, stream))
 
 
 _lock = threading.Lock()

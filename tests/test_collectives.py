@@ -42,10 +42,13 @@ def test_reduce_scatter_driver(target, dtype, mode, alg, P):
         assert_bits_equal(to_numpy(t_in[r], dtype), ins[r], f"input of rank {r} modified")
 
 
-@pytest.mark.parametrize("alg,P", [("ring", 65), ("ring", 100), ("recursive", 128)])
-@pytest.mark.parametrize("mode", ["steps", "faithful"])
+@pytest.mark.parametrize("alg,P", [("ring", 65), ("ring", 100), ("ring", 128), ("recursive", 128), ("recursive", 256)])
+@pytest.mark.parametrize("mode", ["steps", "faithful", "fused"])
 def test_more_ranks_than_one_launch_holds(target, alg, P, mode):
-    """Beyond 64 ranks a step goes out as several launches."""
+    """Beyond 64 ranks a step goes out as several launches; the fused ring
+    order chains folds of at most 64 operands with the running sum as the first
+    operand, the fused halving order runs rounds until groups of 64 remain and
+    finishes each group with one butterfly launch."""
     import torch
     from pccl import kernels
     B, dtype = 21, O.BF16
@@ -58,12 +61,10 @@ def test_more_ranks_than_one_launch_holds(target, alg, P, mode):
     for r in range(P):
         assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"rank {r}")
     g_out = [torch.zeros(P * B, dtype=torch.bfloat16, device=target.device) for _ in range(P)]
-    kernels.all_gather_ranks(g_out, t_out, alg, "steps")
+    kernels.all_gather_ranks(g_out, t_out, alg, "fused" if mode == "fused" else "steps")
     target.sync()
-    for r in (0, P // 2, P - 1):
+    for r in (0, 63, 64, P // 2, P - 1):
         assert_bits_equal(to_numpy(g_out[r], dtype), np.concatenate(want), f"gather rank {r}")
-    with pytest.raises(RuntimeError, match="64 in fused mode"):
-        kernels.reduce_scatter_ranks(t_out, t_in, alg, "fused")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -439,6 +440,50 @@ def test_plans_replay_on_fresh_data(target, mode):
     for r in range(P):
         assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"rank {r}")
         assert_bits_equal(to_numpy(g_out[r], dtype), np.concatenate(want), f"gather rank {r}")
+
+
+@pytest.mark.parametrize("mode", ["fused", "steps"])
+def test_repeated_calls_replay_the_checked_arguments(target, mode):
+    """The ordinary API keeps the checked argument pack of a call and replays it
+    when called again on the same tensor objects; fresh data, a storage swapped
+    under one of the tensors and the death of a tensor are all handled."""
+    import gc
+    import torch
+    from pccl import kernels
+    P, B, dtype = 4, 515, O.F32
+    t_in = [torch.zeros(P * B, device=target.device) for _ in range(P)]
+    t_out = [torch.zeros(B, device=target.device) for _ in range(P)]
+    g_out = [torch.zeros(P * B, device=target.device) for _ in range(P)]
+    work = [torch.empty(P * B, device=target.device) for _ in range(P)]
+    before = len(kernels._PLANS)
+    for seed in (91, 92, 93):
+        ins = make_inputs(P, P * B, dtype, seed=seed)
+        for t, x in zip(t_in, ins):
+            t.copy_(to_torch(x, dtype, target.device))
+        kernels.reduce_scatter_ranks(t_out, t_in, "ring", mode, work)
+        kernels.all_gather_ranks(g_out, t_out, "ring", mode)
+        target.sync()
+        want = O.ring_reduce_scatter(ins, dtype)
+        for r in range(P):
+            assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"seed {seed} rank {r}")
+            assert_bits_equal(to_numpy(g_out[r], dtype), np.concatenate(want), f"seed {seed} gather rank {r}")
+    assert len(kernels._PLANS) == before + 2          # one entry per collective, however often it ran
+    # the same tensor object on another storage: the recorded address no longer matches
+    moved = to_torch(make_inputs(1, P * B, dtype, seed=94)[0], dtype, target.device)
+    t_in[2].set_(moved.untyped_storage(), 0, moved.shape)
+    kernels.reduce_scatter_ranks(t_out, t_in, "ring", mode, work)
+    target.sync()
+    ins[2] = to_numpy(moved, dtype)
+    want = O.ring_reduce_scatter(ins, dtype)
+    for r in range(P):
+        assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"after set_ rank {r}")
+    # a wrong size is still refused although an entry for these objects exists
+    t_out[1].set_(torch.zeros(B + 1, device=target.device).untyped_storage(), 0, (B + 1,))
+    with pytest.raises(RuntimeError, match="block_size"):
+        kernels.reduce_scatter_ranks(t_out, t_in, "ring", mode, work)
+    del t_in, t_out, g_out, work, moved
+    gc.collect()
+    assert len(kernels._PLANS) == before              # entries die with their tensors
 
 
 @pytest.mark.parametrize("rec", [True, False])
