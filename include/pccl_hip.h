@@ -340,7 +340,13 @@ int pccl_hip_probe_mix(const void* const* reads, int nr, void* const* writes,
  *                  move about this many MiB each, a fused reduce over at most
  *                  16 shards as launches 1.5 times as large; 0 = always one
  *                  launch; default 1024.  Copies are always one launch).
- * Returns 0, or PCCL_HIP_EINVAL for an unknown key or value.  Process-wide. */
+ * Returns 0, or PCCL_HIP_EINVAL for an unknown key or value.
+ * The settings are process-wide: besides the per-thread error message, they,
+ * the launch counter below and the per-device address of the built-in scratch
+ * array are the only state the library keeps.  Every value is one atomic word
+ * that a launch reads once, so changing a setting while another thread
+ * launches is safe, but that launch may see either value.  They exist for
+ * measurement; the defaults are what the kernels were tuned to. */
 int pccl_hip_set_tuning(const char* key, long value);
 long pccl_hip_get_tuning(const char* key);
 

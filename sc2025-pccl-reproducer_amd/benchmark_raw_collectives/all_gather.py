@@ -43,6 +43,9 @@ def parse_args(argv=None):
                         help="number of virtual ranks (default: $SLURM_NTASKS or 8)")
     parser.add_argument("--sizes", type=int, nargs="*", default=None, help="output sizes per rank in MB")
     parser.add_argument("--data-dir", default="./data")
+    parser.add_argument("--dump", default=None, metavar="FILE.npz",
+                        help="write the inputs and outputs of every rank for the LAST size of the sweep (raw element "
+                             "bits, one row per rank), so that a checker can recompute them")
     return parser.parse_args(argv)
 
 
@@ -107,6 +110,11 @@ def main(argv=None):
             print("===============================")
             writer.writerow([gpu_count, slurm_job_id, size, unit, time_ms, job_bytes, round(gbps, 1),
                              round(100 * gbps / HBM_PEAK_GBPS, 2)])
+            if args.dump and size == sizes[-1]:
+                bits = torch.int32 if dtype == torch.float32 else torch.int16
+                np.savez(args.dump,
+                         inputs=torch.stack([t.view(bits) for t in inputs]).cpu().numpy(),
+                         outputs=torch.stack([t.view(bits) for t in outputs]).cpu().numpy())
             del inputs, outputs
         if args.test:
             print("All tests passed! PCCL outputs match the concatenation of the inputs!")

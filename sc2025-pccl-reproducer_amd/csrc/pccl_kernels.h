@@ -65,18 +65,36 @@ __device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
   return u;
 }
 
+// own + received in fp32, where `own` is the rank's own block and `received` what
+// its neighbour or partner sent: vectorAdd(a, b) of pccl/src/common.cu:5-19.
+// The sum is commutative except for WHICH payload survives when both operands
+// are NaN: the hardware add keeps the one in its first source, and the
+// reference's compiled kernel has `b` there.  The compiler orders the sources of
+// a plain `own + received` as it likes (it did the opposite here), so the
+// instruction is written out; the host build of this file, which only checks
+// indexing, adds plainly.
+__device__ __forceinline__ float add_own_received(float own, float received) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  float r;
+  asm("v_add_f32 %0, %1, %2" : "=v"(r) : "v"(received), "v"(own));
+  return r;
+#else
+  return own + received;
+#endif
+}
+
 struct OpF32 {
   typedef float elem;
   static constexpr int kPerVec = 4;
   static __device__ __forceinline__ u32x4 add(u32x4 a, u32x4 b) {
     u32x4 r;
-    r.x = __float_as_uint(__uint_as_float(a.x) + __uint_as_float(b.x));
-    r.y = __float_as_uint(__uint_as_float(a.y) + __uint_as_float(b.y));
-    r.z = __float_as_uint(__uint_as_float(a.z) + __uint_as_float(b.z));
-    r.w = __float_as_uint(__uint_as_float(a.w) + __uint_as_float(b.w));
+    r.x = __float_as_uint(add_own_received(__uint_as_float(a.x), __uint_as_float(b.x)));
+    r.y = __float_as_uint(add_own_received(__uint_as_float(a.y), __uint_as_float(b.y)));
+    r.z = __float_as_uint(add_own_received(__uint_as_float(a.z), __uint_as_float(b.z)));
+    r.w = __float_as_uint(add_own_received(__uint_as_float(a.w), __uint_as_float(b.w)));
     return r;
   }
-  static __device__ __forceinline__ elem add1(elem a, elem b) { return a + b; }
+  static __device__ __forceinline__ elem add1(elem a, elem b) { return add_own_received(a, b); }
 };
 
 // Two bf16 values per 32-bit word, element 2i in the low half.
@@ -113,10 +131,17 @@ struct AccF32 {
     f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
   }
   static __device__ __forceinline__ float hop(float a, float b) { return a + b; }
+  // one hop of a ring: the running sum `acc` is what the rank received, x its own block
   template <int L>
   static __device__ __forceinline__ void hop_lanes(float* acc, const float* x) {
 #pragma unroll
-    for (int l = 0; l < L; ++l) acc[l] = acc[l] + x[l];
+    for (int l = 0; l < L; ++l) acc[l] = add_own_received(x[l], acc[l]);
+  }
+  // one round of halving: lo is the rank's own partial sum, hi its partner's
+  template <int L>
+  static __device__ __forceinline__ void join_lanes(float* lo, const float* hi) {
+#pragma unroll
+    for (int l = 0; l < L; ++l) lo[l] = add_own_received(lo[l], hi[l]);
   }
   static __device__ __forceinline__ u32x4 narrow(const float* f) {
     u32x4 r;
@@ -161,6 +186,9 @@ struct AccBF16 {
       for (int l = 0; l < L; ++l) acc[l] = hop(acc[l], x[l]);
     }
   }
+  // NaNs are stored as the canonical pattern, so the two operands' roles do not matter here
+  template <int L>
+  static __device__ __forceinline__ void join_lanes(float* lo, const float* hi) { hop_lanes<L>(lo, hi); }
   static __device__ __forceinline__ u32x4 narrow(const float* f) {
     u32x4 r;
     r.x = (bf16_round_hi(f[0]) >> 16) | bf16_round_hi(f[1]);
@@ -742,7 +770,7 @@ __device__ __forceinline__ void tree_sum(Load& load, int first, float* out) {
     float lo[L], hi[L];
     tree_sum<Acc, K, M, 2 * H, L>(load, first, lo);
     tree_sum<Acc, K, M + H, 2 * H, L>(load, first, hi);
-    Acc::template hop_lanes<L>(lo, hi);
+    Acc::template join_lanes<L>(lo, hi);
 #pragma unroll
     for (int l = 0; l < L; ++l) out[l] = lo[l];
   }

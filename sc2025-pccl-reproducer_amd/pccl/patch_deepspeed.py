@@ -116,24 +116,26 @@ def patched_barrier(self, group=None, async_op=False, device_ids=None):
 def patch_deepspeed(intra_node_pg_size: int, comm: Optional[VirtualComm] = None):
     """Patch DeepSpeed's TorchBackend for the calling rank.
 
-    comm: this rank's world communicator of virtual ranks.  Without it the
-    reference's setting applies (torch.distributed initialised, one process per
-    GPU) and only all_gather / reduce_scatter are rerouted."""
+    comm: this rank's world communicator of virtual ranks; required.  The
+    reference's own setting (no comm: torch.distributed initialised, one
+    process per GPU, an mpi4py outer group, pccl/patch_deepspeed.py:95-110)
+    needs real ranks on several GPUs, which this build does not drive: it is
+    refused here, at patch time, rather than at the first collective."""
+    if comm is None:
+        raise RuntimeError("patch_deepspeed: this build runs on virtual ranks only; pass comm=<this rank's "
+                           "pccl.VirtualComm> (VirtualWorld(P).run(...) hands one to every rank)")
+    if not isinstance(comm, VirtualComm):
+        raise TypeError(f"patch_deepspeed: comm must be a pccl.VirtualComm, got {type(comm)}")
     try:
         from deepspeed.comm.torch import TorchBackend
     except ImportError as e:
         raise RuntimeError("patch_deepspeed needs the deepspeed package") from e
-    if comm is None:
-        assert dist.is_initialized()
-        world_size = dist.get_world_size()
-    else:
-        world_size = comm.Get_size()
+    world_size = comm.Get_size()
     assert world_size % intra_node_pg_size == 0
     build()
     _tls.world = comm
     _tls.pg = ProcessGroups(intra_node_pg_size, world_size // intra_node_pg_size,
-                            inner_group_backend="mpi" if comm is not None else "nccl",
-                            outer_group_backend="mpi", comm=comm)
+                            inner_group_backend="mpi", outer_group_backend="mpi", comm=comm)
     with _patch_lock:
         if getattr(TorchBackend, "_pccl_patched", False):
             return

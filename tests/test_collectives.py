@@ -486,8 +486,12 @@ def test_repeated_calls_replay_the_checked_arguments(target, mode):
     assert len(kernels._PLANS) == before              # entries die with their tensors
 
 
-@pytest.mark.parametrize("rec", [True, False])
-def test_all_reduce(target, rec):
+@pytest.mark.parametrize("rec,kwargs", [(True, {}), (False, {}), (True, {"use_yacl": True}),
+                                        (False, {"use_yacl": True, "use_pccl_cpp_backend": False}),
+                                        (False, {"directly_call_mpi": True})])
+def test_all_reduce(target, rec, kwargs):
+    """The reference's keywords (pccl/all_reduce.py:21-28) are accepted; the
+    direct-MPI route sums in ring order."""
     import torch
     import pccl
     P, n = 4, 4 * 257
@@ -495,7 +499,7 @@ def test_all_reduce(target, rec):
     ins = make_inputs(P, n, dtype, seed=51)
     t = [to_torch(x, dtype, target.device) for x in ins]
     world = pccl.VirtualWorld(P, target.device)
-    world.run(lambda comm: pccl._all_reduce(t[comm.Get_rank()], group=comm, use_rh_and_rd=rec))
+    world.run(lambda comm: pccl._all_reduce(t[comm.Get_rank()], group=comm, use_rh_and_rd=rec, **kwargs))
     target.sync()
     want = O.all_reduce(ins, dtype, "recursive" if rec else "ring")
     for r in range(P):
@@ -590,6 +594,14 @@ def test_patch_deepspeed_routes_world_collectives(target, monkeypatch):
         assert_bits_equal(to_numpy(g_out[r], dtype), np.concatenate(want), f"all_gather rank {r}")
         assert_bits_equal(to_numpy(ar[r], dtype), want_ar[r], f"all_reduce rank {r}")
         assert bool((bc[r] == 3.0).all())
+
+
+def test_patch_deepspeed_without_a_virtual_communicator_is_refused_at_patch_time():
+    from pccl import patch_deepspeed as pd
+    with pytest.raises(RuntimeError, match="virtual ranks only"):
+        pd.patch_deepspeed(2)
+    with pytest.raises(TypeError, match="must be a pccl.VirtualComm"):
+        pd.patch_deepspeed(2, comm=object())
 
 
 def test_patch_deepspeed_without_deepspeed_raises(target):
