@@ -339,7 +339,7 @@ int pccl_hip_probe_mix(const void* const* reads, int nr, void* const* writes,
  *      "launch_mib" (a step of the add kernels goes out as equal launches that
  *                  move about this many MiB each, a fused reduce over at most
  *                  16 shards as launches 1.5 times as large; 0 = always one
- *                  launch; default 1024.  Copies are always one launch).
+ *                  launch; default 768.  Copies are always one launch).
  * Returns 0, or PCCL_HIP_EINVAL for an unknown key or value.
  * The settings are process-wide: besides the per-thread error message, they,
  * the launch counter below and the per-device address of the built-in scratch

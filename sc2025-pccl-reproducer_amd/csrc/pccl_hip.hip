@@ -62,7 +62,7 @@ std::atomic<long> g_unroll_gather{0};  // vectors per thread in the all_gather p
 std::atomic<long> g_gather_strip{-1};  // work items per XCD and strip of the time-blocked gather; 0 = the multicast kernel, -1 = chosen per launch
 std::atomic<long> g_gather_strip_from{-1};  // shortest longest-shard (bytes) the time-blocked gather is chosen for when gather_strip = -1
 std::atomic<unsigned long long> g_launches{0};   // kernel launches issued so far
-std::atomic<long> g_launch_mib{1024};  // traffic per launch of the add kernels, MiB (0 = a step is one launch whatever its size)
+std::atomic<long> g_launch_mib{768};   // traffic per launch of the add kernels, MiB (0 = a step is one launch whatever its size)
 // Non-temporal loads / stores: 1 = always, 0 = never, -1 = by the footprint of
 // the call.  Data that fits the 256 MB Infinity Cache and the L2s is better left
 // cacheable (the next step or call finds it there: a P=8 ring reduce_scatter of
