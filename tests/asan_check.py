@@ -104,4 +104,63 @@ for unroll in (1, 4, 8):
         for k, n in enumerate(lens):
             assert np.array_equal(x[off[k]:off[k] + n], shards[k])
     checked += 1
+# the time-blocked placement kernel (chosen for long shards by default: forced here), every tile count per workgroup
+lib.set_tuning("gather_strip_from", 0)
+cases = [(ug, strip, P, blk) for ug in (0, 1, 8) for strip in (-1, 3) for P in (2, 5) for blk in (17, 4096 + 7, 70001)]
+cases += [(0, -1, 16, 4096 + 7), (2, 1, 3, 1), (0, 160, 2, 70001)]
+for ug, strip, P, blk in cases:
+    lib.set_tuning("unroll_gather", ug)
+    lib.set_tuning("gather_strip", strip)
+    ins = [rng.integers(0, 256, blk, dtype=np.uint8) for _ in range(P)]
+    outs = [np.zeros(P * blk, np.uint8) for _ in range(P)]
+    lib.all_gather_virtual([ptr(o) for o in outs], [ptr(i) for i in ins], blk, "ring", 1)
+    for o in outs:
+        assert np.array_equal(o, np.concatenate(ins))
+    checked += 1
+for ug, strip in ((0, -1), (1, 3), (8, 2)):
+    lib.set_tuning("unroll_gather", ug)
+    lib.set_tuning("gather_strip", strip)
+    outs = [np.zeros(off[-1] + lens[-1], np.uint8) for _ in lens]
+    lib.all_gather_uneven_virtual([ptr(x) for x in outs], [ptr(s) if s.size else 0 for s in shards], lens, off)
+    for x in outs:
+        for k, n in enumerate(lens):
+            assert np.array_equal(x[off[k]:off[k] + n], shards[k])
+    checked += 1
+lib.set_tuning("gather_strip", -1); lib.set_tuning("gather_strip_from", -1); lib.set_tuning("unroll_gather", 0)
+
+# fused modes beyond the ranks of one launch, and the entry point with built-in work buffers
+for alg, P, B in (("ring", 65, 5), ("recursive", 128, 3)):
+    ins = [arr(P * B, O.BF16) for _ in range(P)]
+    want = (O.ring_reduce_scatter if alg == "ring" else O.recursive_halving_reduce_scatter)(ins, O.BF16)
+    outs = [np.zeros(B, np.uint16) for _ in range(P)]
+    work = [np.zeros(P * B, np.uint16) for _ in range(P)]
+    lib.reduce_scatter_virtual([ptr(o) for o in outs], [ptr(i) for i in ins], [ptr(w) for w in work], B, 1, alg, 1)
+    for r in range(P):
+        assert np.array_equal(outs[r], want[r]), (alg, P, r)
+    gouts = [np.zeros(P * B, np.uint16) for _ in range(P)]
+    lib.all_gather_virtual([ptr(g) for g in gouts], [ptr(o) for o in outs], 2 * B, alg, 1)
+    for g in gouts:
+        assert np.array_equal(g, np.concatenate(want))
+    checked += 1
+for alg, P, B in (("ring", 8, 4099), ("recursive", 4, 515), ("ring", 3, 1)):
+    for dtype, code in ((O.F32, 0), (O.BF16, 1)):
+        ins = [arr(P * B, dtype) for _ in range(P)]
+        want = (O.ring_reduce_scatter if alg == "ring" else O.recursive_halving_reduce_scatter)(ins, dtype)
+        outs = [np.zeros(B, ins[0].dtype) for _ in range(P)]
+        lib.reduce_scatter_virtual_noalloc([ptr(o) for o in outs], [ptr(i) for i in ins], B, code, alg)
+        for r in range(P):
+            assert np.array_equal(outs[r].view(np.uint8), want[r].view(np.uint8)), (alg, P, dtype, r)
+        checked += 1
+
+# the measurement probes on exact-size buffers
+for nb in (4096, 4096 * 5 + 16, 70000 // 16 * 16):
+    bufs = [np.zeros(nb, np.uint8) for _ in range(4)]
+    lib.probe_stream(0, ptr(bufs[0]), nb)
+    lib.probe_stream(1, ptr(bufs[1]), nb)
+    for shape in (0, 1):
+        for vec in (1, 2, 4):
+            lib.probe_mix([ptr(bufs[0]), ptr(bufs[1])], [ptr(bufs[2]), ptr(bufs[3])], nb, shape, vec)
+            lib.probe_mix([ptr(bufs[0])], [], nb, shape, vec)
+            lib.probe_mix([], [ptr(bufs[3])], nb, shape, vec)
+            checked += 1
 print(f"ASAN CHECK OK ({checked} cases)")

@@ -74,3 +74,37 @@ def test_noalloc_refuses_what_does_not_fit():
         lib.reduce_scatter_virtual_noalloc([64] * 6, [64] * 6, 8, _native.F32, "recursive")
     # nothing to do: accepted without touching the device
     lib.reduce_scatter_virtual_noalloc([64] * 4, [64] * 4, 0, _native.F32, "ring")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("algorithm", ["ring", "recursive"])
+def test_noalloc_replays_from_a_graph(algorithm):
+    """What the entry point is for: captured into a HIP graph (the set-up call
+    was made outside the capture), it replays with eager work between the
+    replays and gives the oracle's bits on fresh inputs every time."""
+    import torch
+    from pccl import _native, kernels
+    lib = _native.load()
+    dev = "cuda:0"
+    P, B, dtype = 8, 4096 + 24, O.BF16
+    t_in = [to_torch(x, dtype, dev) for x in make_inputs(P, P * B, dtype, seed=11)]
+    t_out = [torch.zeros(B, dtype=torch.bfloat16, device=dev) for _ in range(P)]
+    outs, ins = [t.data_ptr() for t in t_out], [t.data_ptr() for t in t_in]
+    lib.reduce_scatter_virtual_noalloc(outs, ins, B, _native.BF16, algorithm, kernels.stream_handle())
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        lib.reduce_scatter_virtual_noalloc(outs, ins, B, _native.BF16, algorithm, kernels.stream_handle())
+    ref = O.ring_reduce_scatter if algorithm == "ring" else O.recursive_halving_reduce_scatter
+    for rep in range(3):
+        fresh = make_inputs(P, P * B, dtype, seed=100 + rep)
+        for t, x in zip(t_in, fresh):
+            t.copy_(to_torch(x, dtype, dev))
+        for o in t_out:
+            o.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = ref(fresh, dtype)
+        for r in range(P):
+            assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"replay {rep} rank {r}")
