@@ -761,15 +761,24 @@ int gather_place_all(void* const* outputs, int nout, const void* const* inputs, 
   const long unroll_set = g_unroll_gather.load(std::memory_order_relaxed);
   const long pad_set = g_lds_pad_gather.load(std::memory_order_relaxed);
   t.unroll = unroll_set > 0 ? (int)unroll_set : strip > 0 ? 4 : 1;
+  size_t n_local = 0;
+  if (strip > 0) {
+    // work items per shard and XCD, each t.unroll tiles; whole strips
+    const size_t items = (tiles_for(longest, 1) + kXcds * t.unroll - 1) / (kXcds * t.unroll);
+    const bool automatic = g_gather_strip.load(std::memory_order_relaxed) < 0;
+    if (automatic && items + items / 4 + 1 < (size_t)strip) strip = (long)(items + items / 4 + 1);
+    n_local = (items + (size_t)strip - 1) / (size_t)strip * (size_t)strip;
+    // one work item per (shard, output, XCD, item): beyond what a launch counts, the automatic choice
+    // falls back to the multicast kernel, which needs 1/16 of the work items
+    if (n_local > kMaxWorkItems / ((size_t)P * (size_t)nout * kXcds)) {
+      if (!automatic) return check_work_items((size_t)P * (size_t)nout * kXcds, n_local, what);
+      strip = 0;
+      t.unroll = unroll_set > 0 ? (int)unroll_set : 1;
+    }
+  }
   const unsigned lds = (unsigned)(pad_set >= 0 ? pad_set : strip > 0 ? 49152 : 0);
   if (strip > 0) {
     const int U = t.unroll;
-    // work items per shard and XCD, each U tiles; whole strips
-    const size_t items = (tiles_for(longest, 1) + kXcds * U - 1) / (kXcds * U);
-    if (g_gather_strip.load(std::memory_order_relaxed) < 0 && items + items / 4 + 1 < (size_t)strip)
-      strip = (long)(items + items / 4 + 1);
-    const size_t n_local = (items + (size_t)strip - 1) / (size_t)strip * (size_t)strip;
-    if (int rc = check_work_items((size_t)P * (size_t)nout * kXcds, n_local, what)) return rc;
     const bool nts = stream_hint(g_gather_nt.load(), moved);
     hipStream_t st = (hipStream_t)stream;
 #define PCCL_STRIPS(UV)                                                                                              \
