@@ -197,11 +197,14 @@ _PLANS_MAX = 512
 
 
 class _Plan:
-    __slots__ = ("lib", "fn", "args", "ptrs", "lens", "tables", "__weakref__")
+    __slots__ = ("lib", "fn", "args", "ptrs", "lens", "tables", "finals", "__weakref__")
 
 
 def _plan_drop(key):
-    _PLANS.pop(key, None)
+    ent = _PLANS.pop(key, None)
+    if ent is not None:
+        for f in ent.finals:          # the other tensors of the entry need not report their death any more
+            f.detach()
 
 
 def _plan_lookup(key, tensors_a, tensors_b):
@@ -214,21 +217,21 @@ def _plan_lookup(key, tensors_a, tensors_b):
         if ent.fn(*ent.args, stream_handle()):
             raise _native.NativeError(ent.lib.last_error())
         return True
-    _PLANS.pop(key, None)
+    _plan_drop(key)
     return False
 
 
 def _plan_store(key, lib, fn, args, tables, tensors_a, tensors_b, extra=()):
     import weakref
     if len(_PLANS) >= _PLANS_MAX:
-        _PLANS.clear()
+        for k in list(_PLANS):
+            _plan_drop(k)
     ent = _Plan()
     ent.lib, ent.fn, ent.args, ent.tables = lib, fn, args, tables
     ent.ptrs = (*[t.data_ptr() for t in tensors_a], *[t.data_ptr() for t in tensors_b])
     ent.lens = (tensors_a[0].numel(), tensors_b[0].numel())
+    ent.finals = [weakref.finalize(t, _plan_drop, key) for t in (*tensors_a, *tensors_b, *extra)]
     _PLANS[key] = ent
-    for t in (*tensors_a, *tensors_b, *extra):
-        weakref.finalize(t, _plan_drop, key)
 
 
 def reduce_scatter_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[torch.Tensor],

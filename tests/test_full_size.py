@@ -168,6 +168,24 @@ def test_config4_all_gather_p16_128mib_shards(alg, mode):
         assert _same_bits(outs[r], cat), f"rank {r}"
 
 
+@pytest.mark.parametrize("P,shard_bytes", [(64, 8 * MiB), (3, 300 * MiB + 5), (2, (1 << 32) + 4099), (5, 2 * MiB)])
+def test_time_blocked_gather_shapes(P, shard_bytes):
+    """The fused all_gather at shapes around its strips: many short shards (one
+    strip per shard), ragged byte counts, a shard longer than 2^32 bytes, and
+    the shortest shard the time-blocked kernel is chosen for."""
+    import torch
+    from pccl import kernels
+    print(f"time-blocked gather P={P} shard={shard_bytes}", flush=True)
+    g = torch.Generator(device=DEV).manual_seed(P)
+    ins = [torch.randint(0, 256, (shard_bytes,), dtype=torch.uint8, device=DEV, generator=g) for _ in range(P)]
+    outs = [torch.full((P * shard_bytes,), 0x5A, dtype=torch.uint8, device=DEV) for _ in range(P)]
+    kernels.all_gather_ranks(outs, ins, "ring", "fused")
+    torch.cuda.synchronize()
+    for r in range(P):
+        for k in range(P):
+            assert torch.equal(outs[r][k * shard_bytes:(k + 1) * shard_bytes], ins[k]), (r, k)
+
+
 def test_config4_uneven_shards_padded_to_256_bytes():
     import torch
     from pccl import kernels
