@@ -42,6 +42,21 @@ __device__ __forceinline__ void st16(u32x4* p, u32x4 v) {
   else *p = v;
 }
 
+// The same 16 bytes at ANY address.  gfx950 takes vector accesses that are not
+// 16-byte (or even 4-byte) aligned; one that straddles its natural boundary is
+// split into more requests, which is still far ahead of an element-wise loop
+// (measured on MI355X: a bf16 fold of 12 shards whose blocks start at odd
+// multiples of 2 bytes 2.2 -> 5.5 TB/s, an accumulate whose source is one element
+// off the destination's alignment 3.3 -> 6.4, a copy one byte off 1.9 -> 6.4).
+// For an aligned address it is the very same instruction.
+typedef uint32_t u32x4_any __attribute__((ext_vector_type(4), aligned(1)));
+
+template <bool NT>
+__device__ __forceinline__ u32x4 ld16u(const void* p) {
+  if constexpr (NT) return __builtin_nontemporal_load((const u32x4_any*)p);
+  else return *(const u32x4_any*)p;
+}
+
 // Round an fp32 value (given as bits) to bfloat16, ties to even; the result
 // stays in the upper 16 bits so that it is again a valid fp32 operand.
 // NaN becomes the canonical quiet NaN 0x7FC0, as on the host.
@@ -218,21 +233,21 @@ struct AccBF16 {
   }
 };
 
-// How a segment of `n` elements at (dst, a, b) splits into an unaligned head
-// (elements before the first 16-byte boundary), a body of whole 128-bit vectors
-// and a tail.  If the operands do not share one misalignment the whole segment
-// is done element by element (vec == 0).
+// How a segment of `n` elements splits into a head (elements before the first
+// 16-byte boundary of the DESTINATION), a body of whole 128-bit vectors and a
+// tail.  Stores of the body are aligned; the sources are read at whatever
+// alignment they have (ld16u).  A destination that is not even element-aligned,
+// or a segment shorter than one vector, is done element by element (vec == 0).
 struct Split {
   size_t head;   // elements
   size_t vec;    // 16-byte vectors
   size_t tail;   // elements
 };
 
-__device__ __forceinline__ Split split_segment(uintptr_t p0, uintptr_t p1, uintptr_t p2, size_t n,
-                                               unsigned esize) {
+__device__ __forceinline__ Split split_segment(uintptr_t dst, size_t n, unsigned esize) {
   Split s;
-  unsigned mis = (unsigned)(p0 & 15u);
-  if ((p1 & 15u) != mis || (p2 & 15u) != mis || (mis % esize) != 0) {
+  const unsigned mis = (unsigned)(dst & 15u);
+  if ((mis % esize) != 0) {
     s.head = n; s.vec = 0; s.tail = 0;
     return s;
   }
@@ -278,15 +293,15 @@ __device__ __forceinline__ void add_tile(void* dstp, const void* ap, const void*
     }
     return;
   }
-  const Split sp = split_segment((uintptr_t)dstp, (uintptr_t)ap, (uintptr_t)bp, n, sizeof(elem));
+  const Split sp = split_segment((uintptr_t)dstp, n, sizeof(elem));
   elem* de = (elem*)dstp;
   const elem* ae = (const elem*)ap;
   const elem* be = (const elem*)bp;
   const unsigned tid = threadIdx.x;
 
   if (sp.vec == 0) {
-    // no common alignment (or a segment shorter than one vector): scalar path,
-    // each tile takes the element range its vectors would have covered
+    // a segment shorter than one vector: scalar path, each tile takes the
+    // element range its vectors would have covered
     const size_t per_tile = (size_t)kThreads * U * Op::kPerVec;
     size_t lo = tile * per_tile;
     size_t hi = lo + per_tile < sp.head ? lo + per_tile : sp.head;
@@ -295,23 +310,23 @@ __device__ __forceinline__ void add_tile(void* dstp, const void* ap, const void*
   }
 
   u32x4* dv = (u32x4*)(de + sp.head);
-  const u32x4* av = (const u32x4*)(ae + sp.head);
-  const u32x4* bv = (const u32x4*)(be + sp.head);
+  const uint8_t* av = (const uint8_t*)(ae + sp.head);   // the sources may sit at any element alignment
+  const uint8_t* bv = (const uint8_t*)(be + sp.head);
   const size_t base = tile * (size_t)(kThreads * U);
 
   if (base + (size_t)kThreads * U <= sp.vec) {
     u32x4 x[U], y[U];
 #pragma unroll
-    for (int j = 0; j < U; ++j) x[j] = ld16<NTL>(av + base + (size_t)j * kThreads + tid);
+    for (int j = 0; j < U; ++j) x[j] = ld16u<NTL>(av + (base + (size_t)j * kThreads + tid) * 16);
 #pragma unroll
-    for (int j = 0; j < U; ++j) y[j] = ld16<NTL>(bv + base + (size_t)j * kThreads + tid);
+    for (int j = 0; j < U; ++j) y[j] = ld16u<NTL>(bv + (base + (size_t)j * kThreads + tid) * 16);
 #pragma unroll
     for (int j = 0; j < U; ++j) st16<NTS>(dv + base + (size_t)j * kThreads + tid, Op::add(x[j], y[j]));
   } else {
 #pragma unroll
     for (int j = 0; j < U; ++j) {
       size_t v = base + (size_t)j * kThreads + tid;
-      if (v < sp.vec) st16<NTS>(dv + v, Op::add(ld16<NTL>(av + v), ld16<NTL>(bv + v)));
+      if (v < sp.vec) st16<NTS>(dv + v, Op::add(ld16u<NTL>(av + v * 16), ld16u<NTL>(bv + v * 16)));
     }
   }
 
@@ -359,7 +374,7 @@ __device__ __forceinline__ void copy_tile(void* dstp, const void* srcp, size_t n
     }
     return;
   }
-  const Split sp = split_segment((uintptr_t)dstp, (uintptr_t)srcp, (uintptr_t)srcp, nbytes, 1);
+  const Split sp = split_segment((uintptr_t)dstp, nbytes, 1);
   uint8_t* d8 = (uint8_t*)dstp;
   const uint8_t* s8 = (const uint8_t*)srcp;
   const unsigned tid = threadIdx.x;
@@ -386,18 +401,18 @@ __device__ __forceinline__ void copy_tile(void* dstp, const void* srcp, size_t n
   }
 
   u32x4* dv = (u32x4*)(d8 + sp.head);
-  const u32x4* sv = (const u32x4*)(s8 + sp.head);
+  const uint8_t* sv = s8 + sp.head;                      // any alignment
   if (copy_vec<U>(tile, U - 1) < sp.vec) {
     u32x4 x[U];
 #pragma unroll
-    for (int j = 0; j < U; ++j) x[j] = ld16<NTL>(sv + copy_vec<U>(tile, j));
+    for (int j = 0; j < U; ++j) x[j] = ld16u<NTL>(sv + copy_vec<U>(tile, j) * 16);
 #pragma unroll
     for (int j = 0; j < U; ++j) st16<NTS>(dv + copy_vec<U>(tile, j), x[j]);
   } else {
 #pragma unroll
     for (int j = 0; j < U; ++j) {
       const size_t v = copy_vec<U>(tile, j);
-      if (v < sp.vec) st16<NTS>(dv + v, ld16<NTL>(sv + v));
+      if (v < sp.vec) st16<NTS>(dv + v, ld16u<NTL>(sv + v * 16));
     }
   }
   if (tile == 0) {
@@ -894,9 +909,9 @@ __device__ __forceinline__ void fold_shards(Load&& load, int k, int g, int first
 // Fused k-way reduce, one pass: output j = fold over the k shards of
 // shard[.][eoff[j] + i], i < n, starting the schedule at shard
 // (first0 + j) mod k (or, for the two-level ring, at the inner and outer
-// successors of j).  The vector path needs 16-byte aligned operands;
-// otherwise (and for the last n % kPerVec elements) elements go one by one
-// through the same fold.
+// successors of j).  The vector path needs a 16-byte aligned output (the shards
+// may start anywhere); otherwise (and for the last n % kPerVec elements)
+// elements go one by one through the same fold.
 template <class Acc, int K, int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int g, int nout,
                                                           size_t n, int first0,
@@ -917,9 +932,9 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
     const size_t eoff = t.eoff[j];
     elem* out = (elem*)t.out[j];
 
-    bool aligned = (((uintptr_t)out) & 15u) == 0;
-    for (int q = 0; q < k; ++q)
-      aligned = aligned && (((uintptr_t)((const elem*)t.shard[q] + eoff)) & 15u) == 0;
+    // stores are aligned vectors, so the output must start on a 16-byte boundary;
+    // the shards are read at whatever element alignment block eoff has (ld16u)
+    const bool aligned = (((uintptr_t)out) & 15u) == 0;
     const size_t nvec = aligned ? n / Op::kPerVec : 0;
     const size_t base = tile * (size_t)(kThreads * U);
 
@@ -943,7 +958,7 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
               // pointers are fetched up front and spill out of the scalar registers
               asm volatile("" : "+s"(q));
 #endif
-              x[r] = ld16<NTL>((const u32x4*)((const uint8_t*)t.shard[q] + wg_byte + lane_byte));
+              x[r] = ld16u<NTL>((const uint8_t*)t.shard[q] + wg_byte + lane_byte);
             }
           };
           tree_vec<Acc, K / G, 0, 1, G>(group_load, part);
@@ -959,7 +974,7 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
         float acc[L];
         fold_shards<Acc, K, L>(
             [&](int q, float* f) {
-              Acc::widen(ld16<NTL>((const u32x4*)((const uint8_t*)t.shard[q] + wg_byte + lane_byte)), f);
+              Acc::widen(ld16u<NTL>((const uint8_t*)t.shard[q] + wg_byte + lane_byte), f);
             },
             k, g, first, first_outer, acc);
         st16<NTS>((u32x4*)out + v, Acc::narrow(acc));
