@@ -46,8 +46,8 @@ extern "C" {
 #define PCCL_HIP_ABI_VERSION 1
 
 /* Largest number of segments / shards one LAUNCH takes (their pointers travel
- * in the kernel arguments): the limit of the batched kernels, of the uneven
- * all_gather and of the 2-D entry points. */
+ * in the kernel arguments): the limit of the batched kernels and of the 2-D
+ * entry points. */
 #define PCCL_HIP_MAX_RANKS 64
 
 /* Largest number of virtual ranks of pccl_hip_reduce_scatter_virtual /
@@ -248,8 +248,10 @@ int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs,
 
 /* Uneven all_gather: shard k has nbytes[k] bytes and lands at byte offset
  * dst_off[k] of every output (the caller chooses offsets, e.g. each shard
- * padded to a multiple of 256 bytes).  One launch places all P*P segments.
- * Not a reference feature (it requires equal shards, pccl/src/pccl.cpp:111-116). */
+ * padded to a multiple of 256 bytes).  One launch places all P*P segments
+ * (one per 64 shards and 64 outputs beyond PCCL_HIP_MAX_RANKS ranks).
+ * 1 <= P <= PCCL_HIP_MAX_VIRTUAL_RANKS.  Not a reference feature (it requires
+ * equal shards, pccl/src/pccl.cpp:111-116). */
 int pccl_hip_all_gather_uneven_virtual(void* const* outputs,
                                        const void* const* inputs,
                                        const size_t* nbytes,

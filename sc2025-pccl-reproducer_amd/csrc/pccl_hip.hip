@@ -822,11 +822,23 @@ int pccl_hip_all_gather_uneven_virtual(void* const* outputs, const void* const* 
                                        const size_t* nbytes, const size_t* dst_off, int P,
                                        void* stream) {
   const char* what = "pccl_hip_all_gather_uneven_virtual";
-  if (P < 1 || P > kMaxSeg) return fail(PCCL_HIP_EINVAL, "%s: P = %d outside [1, %d]", what, P, kMaxSeg);
+  if (P < 1 || P > kMaxVirtualRanks)
+    return fail(PCCL_HIP_EINVAL, "%s: P = %d outside [1, %d]", what, P, kMaxVirtualRanks);
   if (!nbytes || !dst_off) return fail(PCCL_HIP_EINVAL, "%s: NULL size table", what);
   if (int rc = check_table((const void* const*)outputs, P, what, "outputs")) return rc;
   if (!inputs) return fail(PCCL_HIP_EINVAL, "%s: inputs is NULL", what);
-  return gather_place_all(outputs, P, inputs, nbytes, dst_off, P, stream, what);
+  size_t total = 0;
+  for (int k = 0; k < P; ++k) total += nbytes[k];
+  CallBytes footprint(((size_t)P + 1) * total);   // P shards and P outputs holding all of them
+  // one launch places up to kMaxSeg shards into up to kMaxSeg outputs
+  for (int k0 = 0; k0 < P; k0 += kMaxSeg) {
+    const int nk = P - k0 < kMaxSeg ? P - k0 : kMaxSeg;
+    for (int r0 = 0; r0 < P; r0 += kMaxSeg) {
+      const int nr = P - r0 < kMaxSeg ? P - r0 : kMaxSeg;
+      if (int rc = gather_place_all(outputs + r0, nr, inputs + k0, nbytes + k0, dst_off + k0, nk, stream, what)) return rc;
+    }
+  }
+  return PCCL_HIP_OK;
 }
 
 }  // extern "C"

@@ -172,6 +172,23 @@ def test_all_gather_uneven_padded_to_256(target):
     assert torch.equal(got, torch.cat([as_bytes(t) for t in t_in]))
 
 
+def test_all_gather_uneven_more_ranks_than_one_launch_holds(target):
+    import torch
+    from pccl import kernels
+    P = 70
+    rng = np.random.default_rng(70)
+    nbytes = [int(x) for x in rng.integers(0, 3000, P)]
+    t_in = [torch.from_numpy(rng.integers(0, 256, n, dtype=np.uint8)).to(target.device) for n in nbytes]
+    off = kernels.padded_offsets(nbytes, 256)
+    total = off[-1] + nbytes[-1]
+    t_out = [torch.full((total,), 0x5A, dtype=torch.uint8, device=target.device) for _ in range(P)]
+    kernels.all_gather_uneven_ranks(t_out, t_in, off)
+    target.sync()
+    want = O.uneven_all_gather([t.cpu().numpy() for t in t_in], off, total, fill=0x5A)
+    for r in (0, 63, 64, 69):
+        assert np.array_equal(t_out[r].cpu().numpy(), want[r]), f"rank {r}"
+
+
 @pytest.mark.parametrize("P", [1, 3, 5, 16])
 @pytest.mark.parametrize("split,strip", [(0, 0), (1, 0), (2, 0), (3, 0), (64, 0), (0, 1), (0, 2), (0, 256), (0, -1)])
 @pytest.mark.parametrize("unroll,nt", [(1, 1), (4, 0)])
