@@ -631,29 +631,31 @@ __global__ __launch_bounds__(kThreads) void k_gather_strips(GatherArgs t, int P,
     if (tile0 != 0 && tile0 * kTileBytes >= nb + 16) continue;
     const uint8_t* src = (const uint8_t*)t.ins[k];
     uint8_t* dst = (uint8_t*)t.outs[r] + t.dst_off[k];
-    const size_t nvec = nb / 16;
-    if (((((uintptr_t)src) | ((uintptr_t)dst)) & 15u) == 0) {
-      const size_t v0 = tile0 * kThreads + tid;
-      if (v0 + (size_t)(U - 1) * kXcds * kThreads < nvec) {
-        u32x4 xv[U];
+    // head up to the destination's first 16-byte boundary, aligned vector stores behind
+    // it, the source read at whatever alignment that leaves it (ld16u), then the tail
+    size_t head = (16u - (unsigned)((uintptr_t)dst & 15u)) & 15u;
+    if (head > nb) head = nb;
+    const size_t nvec = (nb - head) / 16;
+    u32x4* dv = (u32x4*)(dst + head);
+    const uint8_t* sv = src + head;
+    const size_t v0 = tile0 * kThreads + tid;
+    if (v0 + (size_t)(U - 1) * kXcds * kThreads < nvec) {
+      u32x4 xv[U];
 #pragma unroll
-        for (int j = 0; j < U; ++j) xv[j] = ld16<NTL>((const u32x4*)src + v0 + (size_t)j * kXcds * kThreads);
+      for (int j = 0; j < U; ++j) xv[j] = ld16u<NTL>(sv + (v0 + (size_t)j * kXcds * kThreads) * 16);
 #pragma unroll
-        for (int j = 0; j < U; ++j) st16<NTS>((u32x4*)dst + v0 + (size_t)j * kXcds * kThreads, xv[j]);
-      } else {
-#pragma unroll
-        for (int j = 0; j < U; ++j) {
-          const size_t v = v0 + (size_t)j * kXcds * kThreads;
-          if (v < nvec) st16<NTS>((u32x4*)dst + v, ld16<NTL>((const u32x4*)src + v));
-        }
-      }
-      if (tile0 == 0 && tid < nb - nvec * 16) dst[nvec * 16 + tid] = src[nvec * 16 + tid];   // the last nb % 16 bytes
+      for (int j = 0; j < U; ++j) st16<NTS>(dv + v0 + (size_t)j * kXcds * kThreads, xv[j]);
     } else {
 #pragma unroll
       for (int j = 0; j < U; ++j) {
-        const size_t tile = tile0 + (size_t)j * kXcds;
-        if (tile == 0 || tile * kTileBytes < nb + 16) copy_tile<1, NTL, NTS>(dst, src, nb, tile);
+        const size_t v = v0 + (size_t)j * kXcds * kThreads;
+        if (v < nvec) st16<NTS>(dv + v, ld16u<NTL>(sv + v * 16));
       }
+    }
+    if (tile0 == 0) {   // at most 15 bytes on either side of the body
+      if (tid < head) dst[tid] = src[tid];
+      const size_t done = head + nvec * 16;
+      if (tid >= 64 && done + (tid - 64) < nb) dst[done + (tid - 64)] = src[done + (tid - 64)];
     }
   }
 }
