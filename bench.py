@@ -909,6 +909,22 @@ def main():
     head_name = "cfg2" if everything else args.workload
     head_mode = (args.mode or default_mode(head_name)) if not everything else "steps"
     want_modes = [head_mode]
+    rows, all_ok = [], True
+    sub_steps, sub_warm = min(args.steps, 10), min(args.warmup, 3)
+
+    def add_row(name, mode, step_fn, info_):
+        nonlocal all_ok
+        r, _, _, _, _ = run_row(name, mode, step_fn, info_, sub_steps, sub_warm, lib, verify=not args.no_verify)
+        rows.append(r)
+        all_ok = all_ok and r["verified"] in (None, True)
+
+    def run_group(name):
+        group = build_workloads(name, [m for n, m in ALL_ROWS if n == name], args.scale, device)
+        for m in group:
+            add_row(name, m, *group[m])
+        del group
+        torch.cuda.empty_cache()
+
     if everything:
         want_modes += [m for n, m in ALL_ROWS if n == head_name and m != head_mode]
     built = build_workloads(head_name, want_modes, args.scale, device)
@@ -939,33 +955,18 @@ def main():
             roof["traffic_note"] = ("HBM bytes per launch from the rocprofv3 FETCH_SIZE/WRITE_SIZE runs summarised in "
                                     "profiles/ (same kernel sources, default tuning, full size); not measured in this run")
 
-    rows, all_ok = [], ok in (None, True)
+    all_ok = all_ok and ok in (None, True)
     extra = {}
     if everything:
-        sub_steps, sub_warm = min(args.steps, 10), min(args.warmup, 3)
-
-        def add_row(name, mode, step_fn, info_):
-            nonlocal all_ok
-            r, _, _, _, _ = run_row(name, mode, step_fn, info_, sub_steps, sub_warm, lib, verify=not args.no_verify)
-            rows.append(r)
-            all_ok = all_ok and r["verified"] in (None, True)
-
         for m in want_modes[1:]:
             add_row(head_name, m, *built[m])
         del built, step
         info = {k: v for k, v in info.items() if k != "verify"}
         torch.cuda.empty_cache()
-        todo = {}
-        for n, m in ALL_ROWS:
-            if n != head_name:
-                todo.setdefault(n, []).append(m)
-        for n, modes in todo.items():
-            group = build_workloads(n, modes, args.scale, device)
-            for m in modes:
-                add_row(n, m, *group[m])
-            del group
-            torch.cuda.empty_cache()
-        rows.sort(key=lambda r: [x for x, _ in ALL_ROWS].index(r["workload"]))
+        for name in dict.fromkeys(n for n, _ in ALL_ROWS):
+            if name != head_name:
+                run_group(name)
+        rows.sort(key=lambda r: ALL_ROWS.index((r["workload"], r["mode"])))
         extra["latency_us"] = latency_sweep(50, 10, device)
         extra["ceilings"] = ceilings(10, 3, device)
         torch.cuda.empty_cache()
