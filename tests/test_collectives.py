@@ -472,7 +472,8 @@ def test_repeated_calls_replay_the_checked_arguments(target, mode):
     t_out = [torch.zeros(B, device=target.device) for _ in range(P)]
     g_out = [torch.zeros(P * B, device=target.device) for _ in range(P)]
     work = [torch.empty(P * B, device=target.device) for _ in range(P)]
-    before = len(kernels._PLANS)
+    gc.collect()
+    before = set(kernels._PLANS)                      # entries of tensors other tests still hold
     for seed in (91, 92, 93):
         ins = make_inputs(P, P * B, dtype, seed=seed)
         for t, x in zip(t_in, ins):
@@ -484,7 +485,8 @@ def test_repeated_calls_replay_the_checked_arguments(target, mode):
         for r in range(P):
             assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"seed {seed} rank {r}")
             assert_bits_equal(to_numpy(g_out[r], dtype), np.concatenate(want), f"seed {seed} gather rank {r}")
-    assert len(kernels._PLANS) == before + 2          # one entry per collective, however often it ran
+    mine = set(kernels._PLANS) - before
+    assert len(mine) == 2                             # one entry per collective, however often it ran
     # the same tensor object on another storage: the recorded address no longer matches
     moved = to_torch(make_inputs(1, P * B, dtype, seed=94)[0], dtype, target.device)
     t_in[2].set_(moved.untyped_storage(), 0, moved.shape)
@@ -500,7 +502,7 @@ def test_repeated_calls_replay_the_checked_arguments(target, mode):
         kernels.reduce_scatter_ranks(t_out, t_in, "ring", mode, work)
     del t_in, t_out, g_out, work, moved
     gc.collect()
-    assert len(kernels._PLANS) == before              # entries die with their tensors
+    assert not (set(kernels._PLANS) & mine)           # entries die with their tensors
 
 
 @pytest.mark.parametrize("rec,kwargs", [(True, {}), (False, {}), (True, {"use_yacl": True}),
