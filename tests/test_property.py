@@ -85,3 +85,78 @@ def test_2d_random_shapes(cpu, intra, inter, m, bf16, rec, mode, seed):
     kernels.all_gather_2d_ranks(g_out, t_out, intra, inter, alg, mode)
     for w in range(W):
         assert_bits_equal(to_numpy(g_out[w], dtype), np.concatenate(want), f"gather rank {w}")
+
+
+@settings(**SETTINGS)
+@given(P=st.integers(1, 9), nmax=st.integers(1, 40000), strip=st.sampled_from([-1, 1, 2, 5, 160]),
+       unroll=st.sampled_from([0, 1, 2, 4, 8]), in_shift=st.integers(0, 15), out_shift=st.integers(0, 15),
+       gap=st.integers(0, 33), seed=st.integers(0, 2 ** 16))
+def test_time_blocked_gather_random_shapes(cpu, P, nmax, strip, unroll, in_shift, out_shift, gap, seed):
+    """The time-blocked placement kernel on shards of random (also zero) lengths at
+    random byte alignments of sources, outputs and offsets: every shard lands where
+    it should and nothing else is touched."""
+    import torch
+    lib = cpu.native
+    keys = ("gather_strip", "gather_strip_from", "unroll_gather")
+    saved = {k: lib.get_tuning(k) for k in keys}
+    rng = np.random.default_rng(seed)
+    nbytes = [int(x) for x in rng.integers(0, nmax + 1, P)]
+    shards = [rng.integers(0, 256, n, dtype=np.uint8) for n in nbytes]
+    off, o = [], 0
+    for n in nbytes:
+        off.append(o)
+        o += n + gap                                   # byte offsets of any alignment, `gap` untouched bytes between
+    total = o
+    big_in = [torch.from_numpy(np.concatenate([np.zeros(in_shift, np.uint8), s])) for s in shards]
+    t_in = [b[in_shift:] for b in big_in]
+    big_out = [torch.full((total + 32,), 0xA5, dtype=torch.uint8) for _ in range(P)]
+    t_out = [b[out_shift:out_shift + total] for b in big_out]
+    try:
+        lib.set_tuning("gather_strip", strip)
+        lib.set_tuning("gather_strip_from", 0)
+        lib.set_tuning("unroll_gather", unroll)
+        lib.all_gather_uneven_virtual([t.data_ptr() for t in t_out], [t.data_ptr() if t.numel() else 0 for t in t_in],
+                                      nbytes, off, 0)
+    finally:
+        for k, v in saved.items():
+            lib.set_tuning(k, v)
+    want = np.full(total + 32, 0xA5, np.uint8)
+    for k in range(P):
+        want[out_shift + off[k]:out_shift + off[k] + nbytes[k]] = shards[k]
+    for r in range(P):
+        assert np.array_equal(big_out[r].numpy(), want), f"rank {r}"
+
+
+@settings(**SETTINGS)
+@given(n=st.integers(1, 20000), bf16=st.booleans(), sd=st.integers(0, 7), sa=st.integers(0, 7), sb=st.integers(0, 7),
+       k=st.integers(2, 9), seed=st.integers(0, 2 ** 16))
+def test_differently_aligned_operands(cpu, n, bf16, sd, sa, sb, k, seed):
+    """dst, a and b (and the shards of a fold) each at its own element alignment:
+    aligned vector stores, sources read wherever they lie; the oracle's bits and
+    nothing written outside dst."""
+    import torch
+    lib = cpu.native
+    dtype = O.BF16 if bf16 else O.F32
+    code = 1 if bf16 else 0
+    td = torch.bfloat16 if bf16 else torch.float32
+    xs = make_inputs(k, n, dtype, seed=seed)
+    bufs = [torch.zeros(n + 8, dtype=td) for _ in range(k)]
+    shifts = [(sa + 3 * q) % 8 for q in range(k)]
+    shifts[1] = sb
+    views = []
+    for q in range(k):
+        v = bufs[q][shifts[q]:shifts[q] + n]
+        v.copy_(to_torch(xs[q], dtype, "cpu"))
+        views.append(v)
+    out_big = torch.zeros(n + 8, dtype=td)
+    out = out_big[sd:sd + n]
+    lib.add(out.data_ptr(), views[0].data_ptr(), views[1].data_ptr(), n, code, 0)
+    assert_bits_equal(to_numpy(out.clone(), dtype), O.vector_add(xs[0], xs[1], dtype), "add")
+    assert not out_big[:sd].float().abs().sum() and not out_big[sd + n:].float().abs().sum()
+    out_big.zero_()
+    lib.reduce_kway(out.data_ptr(), [v.data_ptr() for v in views], n, code, 0, 0, True, 0)
+    want = xs[0]
+    for q in range(1, k):
+        want = O.vector_add(want, xs[q], dtype)
+    assert_bits_equal(to_numpy(out.clone(), dtype), want, "fold")
+    assert not out_big[:sd].float().abs().sum() and not out_big[sd + n:].float().abs().sum()
