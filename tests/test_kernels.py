@@ -133,6 +133,41 @@ def test_reduce_kway_matches_sequential_hops(target, dtype, k, order):
     assert_bits_equal(to_numpy(out, dtype), want, "reduce_kway")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("order,k", [("ring", 5), ("ring", 17), ("halving", 4), ("halving", 16)])
+@pytest.mark.parametrize("out_shift", [0, 3])
+def test_reduce_kway_shards_at_any_alignment(target, dtype, order, k, out_shift):
+    """Every shard at its own element alignment (the fold reads 16-byte vectors
+    wherever they lie), the output aligned (vector stores) or not (elements)."""
+    import torch
+    n = 70001
+    shards = make_inputs(k, n, dtype, seed=60 + k)
+    shifts = [(3 * q + 1) % 8 for q in range(k)]
+    bufs = [to_torch(np.concatenate([np.zeros(sh, x.dtype), x, np.zeros(8 - sh, x.dtype)]), dtype, target.device)
+            for x, sh in zip(shards, shifts)]
+    ts = [b[sh:sh + n] for b, sh in zip(bufs, shifts)]
+    out_big = torch.zeros(n + 8, dtype=ts[0].dtype, device=target.device)
+    out = out_big[out_shift:out_shift + n]
+    first = 2 % k
+    target.native.reduce_kway(out.data_ptr(), [t.data_ptr() for t in ts], n, CODE[dtype],
+                              0 if order == "ring" else 1, first, True, target.stream())
+    target.sync()
+    if order == "ring":
+        want = shards[first]
+        for t in range(1, k):
+            want = O.vector_add(want, shards[(first + t) % k], dtype)
+    else:
+        v = [shards[first ^ m] for m in range(k)]
+        h = k // 2
+        while h >= 1:
+            for m in range(h):
+                v[m] = O.vector_add(v[m], v[m + h], dtype)
+            h //= 2
+        want = v[0]
+    assert_bits_equal(to_numpy(out.clone(), dtype), want, "fold of unaligned shards")
+    assert not out_big[:out_shift].float().abs().sum() and not out_big[out_shift + n:].float().abs().sum()
+
+
 def test_reduce_kway_bf16_single_rounding(target):
     """per_hop_round=0: fp32 partial sums, one rounding at the end (within 1 ulp
     of the per-hop result per hop; here checked exactly against numpy)."""
