@@ -911,9 +911,8 @@ __device__ __forceinline__ void fold_shards(Load&& load, int k, int g, int first
 // Fused k-way reduce, one pass: output j = fold over the k shards of
 // shard[.][eoff[j] + i], i < n, starting the schedule at shard
 // (first0 + j) mod k (or, for the two-level ring, at the inner and outer
-// successors of j).  The vector path needs a 16-byte aligned output (the shards
-// may start anywhere); otherwise (and for the last n % kPerVec elements)
-// elements go one by one through the same fold.
+// successors of j).  Output and shards may start at any element alignment;
+// the few elements around the vector body go one by one through the same fold.
 template <class Acc, int K, int U, bool NTL, bool NTS>
 __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int g, int nout,
                                                           size_t n, int first0,
@@ -934,10 +933,13 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
     const size_t eoff = t.eoff[j];
     elem* out = (elem*)t.out[j];
 
-    // stores are aligned vectors, so the output must start on a 16-byte boundary;
-    // the shards are read at whatever element alignment block eoff has (ld16u)
-    const bool aligned = (((uintptr_t)out) & 15u) == 0;
-    const size_t nvec = aligned ? n / Op::kPerVec : 0;
+    // The elements up to the output's first 16-byte boundary (head) and those behind
+    // its last whole vector (tail) go one by one, the body as aligned vector stores;
+    // the shards are read at whatever element alignment that leaves them (ld16u).
+    const unsigned mis = (unsigned)((uintptr_t)out & 15u);
+    size_t head = (mis % sizeof(elem)) == 0 ? ((16u - mis) & 15u) / sizeof(elem) : n;
+    if (head > n) head = n;
+    const size_t nvec = (n - head) / Op::kPerVec;
     const size_t base = tile * (size_t)(kThreads * U);
 
 #pragma unroll
@@ -945,7 +947,7 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
       const size_t v = base + (size_t)u * kThreads + tid;
       // an address is a workgroup-uniform 64-bit base plus a 32-bit lane offset:
       // the unrolled folds then need no vector registers for their k addresses
-      const size_t wg_byte = eoff * sizeof(elem) + (base + (size_t)u * kThreads) * 16;
+      const size_t wg_byte = (eoff + head) * sizeof(elem) + (base + (size_t)u * kThreads) * 16;
       const uint32_t lane_byte = tid * 16u;
       if constexpr (K >= 16 && Acc::kPacked) {
         if (v < nvec) {
@@ -969,7 +971,7 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
 #pragma unroll
             for (int r = 0; r < h; ++r) part[r] = Acc::add_vec(part[r], part[r + h]);
           }
-          st16<NTS>((u32x4*)out + v, Acc::settle(part[0]));
+          st16<NTS>((u32x4*)(out + head) + v, Acc::settle(part[0]));
         }
       } else
       if (v < nvec) {
@@ -979,21 +981,15 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
               Acc::widen(ld16u<NTL>((const uint8_t*)t.shard[q] + wg_byte + lane_byte), f);
             },
             k, g, first, first_outer, acc);
-        st16<NTS>((u32x4*)out + v, Acc::narrow(acc));
+        st16<NTS>((u32x4*)(out + head) + v, Acc::narrow(acc));
       }
     }
 
-    // scalar remainder: the tail of an aligned segment (tile 0), or everything
-    size_t lo, hi;
-    if (aligned) {
-      lo = nvec * Op::kPerVec;
-      hi = tile == 0 ? n : lo;
-    } else {
-      const size_t per_tile = (size_t)kThreads * U * Op::kPerVec;
-      lo = tile * per_tile;
-      hi = lo + per_tile < n ? lo + per_tile : n;
-    }
-    for (size_t i = lo + tid; i < hi; i += kThreads) {
+    // head and tail, by the first tile of the output
+    const size_t body_end = head + nvec * Op::kPerVec;
+    const size_t loose = tile == 0 ? head + (n - body_end) : 0;
+    for (size_t e = tid; e < loose; e += kThreads) {
+      const size_t i = e < head ? e : body_end + (e - head);
       float acc1[1];
       fold_shards<Acc, K, 1>(
           [&](int q, float* f) {
