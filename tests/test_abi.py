@@ -118,3 +118,14 @@ def test_cpu_tensors_are_rejected():
         kernels.accumulate(a, a.clone())
     with pytest.raises(RuntimeError, match="must reside on the GPU"):
         kernels.reduce_scatter_ranks([torch.zeros(4)] * 2, [torch.zeros(8)] * 2, "ring")
+
+
+@pytest.mark.gpu
+def test_library_called_from_plain_c():
+    """csrc/examples/call_from_c.c, built with gcc against include/pccl_hip.h: accumulate and a
+    ring reduce_scatter (per-step, fused, built-in work buffers) from C, checked there against
+    the host's left fold bit for bit."""
+    exe = os.path.join(ROOT, "sc2025-pccl-reproducer_amd", "csrc", "build", "call_from_c")
+    assert os.path.exists(exe), "not built: make -C sc2025-pccl-reproducer_amd/csrc example"
+    p = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0 and p.stdout.strip() == "OK", (p.returncode, p.stdout, p.stderr)
