@@ -525,7 +525,8 @@ def profiled_traffic(workload, mode, kernel, lib, scale):
     taken with these kernel sources, the default tuning and the full size."""
     path = os.path.join(ROOT, "profiles", "traffic.json")
     try:
-        table = json.load(open(path))
+        with open(path) as fh:
+            table = json.load(fh)
     except Exception:                                         # noqa: BLE001
         return None, "no profiles/traffic.json"
     entry = table.get("entries", {}).get(f"{workload}:{mode}:{kernel}")
