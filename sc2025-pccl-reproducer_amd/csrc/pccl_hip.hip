@@ -57,7 +57,7 @@ std::atomic<long> g_lds_pad_copy{0};   // copy kernels
 std::atomic<long> g_lds_pad_kway{-1};  // fused reduce; -1 = chosen per launch (see launch_kway)
 std::atomic<long> g_lds_pad_gather{-1}; // all_gather placement kernels; -1 = chosen per launch
 std::atomic<long> g_gather_split{0};   // groups of outputs per shard tile in the multicast gather; 0 = four outputs a group
-std::atomic<long> g_gather_nt{-1};     // non-temporal stores in the multicast gather (-1: by footprint, like nt_store)
+std::atomic<long> g_gather_nt{-1};     // non-temporal stores in the all_gather placement kernels (-1: by footprint, like nt_store)
 std::atomic<long> g_unroll_gather{0};  // vectors per thread in the all_gather placement kernels; 0 = chosen per launch
 std::atomic<long> g_gather_strip{-1};  // work items per XCD and strip of the time-blocked gather; 0 = the multicast kernel, -1 = chosen per launch
 std::atomic<long> g_gather_strip_from{-1};  // shortest longest-shard (bytes) the time-blocked gather is chosen for when gather_strip = -1
@@ -749,9 +749,10 @@ int gather_place_all(void* const* outputs, int nout, const void* const* inputs, 
   // the latency of its load, 5.4 TB/s); strips of 160 work items = 2.5 MiB per XCD
   // (beyond the 4 MiB of an L2 the re-reads miss: 3.7 TB/s); three workgroups per
   // CU (48 KiB of unused LDS each, +1 %).  A strip that divides the shard exactly
-  // is 5-15 % slower than one a quarter longer (the two outputs an XCD writes
-  // around a change of output then lie a power of two apart), so short shards get
-  // strips a quarter longer than their work items.
+  // is 5-15 % slower than a longer one (the two outputs an XCD writes around a
+  // change of output then lie a power of two apart); for shards shorter than a
+  // strip, strips of twice their work items (every other slot an empty workgroup)
+  // measured 2-5 % ahead of strips a quarter longer, three times are slower.
   long strip = g_gather_strip.load(std::memory_order_relaxed);
   if (strip < 0) {
     long from = g_gather_strip_from.load(std::memory_order_relaxed);
@@ -766,7 +767,7 @@ int gather_place_all(void* const* outputs, int nout, const void* const* inputs, 
     // work items per shard and XCD, each t.unroll tiles; whole strips
     const size_t items = (tiles_for(longest, 1) + kXcds * t.unroll - 1) / (kXcds * t.unroll);
     const bool automatic = g_gather_strip.load(std::memory_order_relaxed) < 0;
-    if (automatic && items + items / 4 + 1 < (size_t)strip) strip = (long)(items + items / 4 + 1);
+    if (automatic && 2 * items + 1 < (size_t)strip) strip = (long)(2 * items + 1);
     n_local = (items + (size_t)strip - 1) / (size_t)strip * (size_t)strip;
     // one work item per (shard, output, XCD, item): beyond what a launch counts, the automatic choice
     // falls back to the multicast kernel, which needs 1/16 of the work items
