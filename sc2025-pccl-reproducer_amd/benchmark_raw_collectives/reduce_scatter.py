@@ -6,8 +6,9 @@ reference (benchmark_raw_collectives/reduce_scatter.py) on one MI355X.
            --library pccl --pccl-recursive-alg --test [--world-size 8] [--dtype bf16]
 
 Same flags, size sweep (1 .. 1024 MB of input per rank), timing convention and
-CSV layout as the reference; the CSV gains the algorithmic bytes of the job, the
-GB/s they imply and the share of the 8 TB/s HBM peak.  `--library xccl`
+CSV layout as the reference; the CSV gains the bytes the job moves in the execution
+mode in use (one fused pass by default, $PCCL_VIRTUAL_MODE=steps for the per-step
+replay), the GB/s they imply and the share of the 8 TB/s HBM peak.  `--library xccl`
 (torch.distributed) needs real process groups and is not available on virtual
 ranks.  Unlike the reference (benchmark_raw_collectives/reduce_scatter.py:95 forces
 use_rh=True), `--pccl-recursive-alg` really selects the algorithm here.
@@ -23,7 +24,7 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(HERE))
 
-from pccl import ProcessGroups, VirtualWorld, reduce_scatter_2D, _reduce_scatter  # noqa: E402
+from pccl import ProcessGroups, VirtualWorld, kernels, reduce_scatter_2D, _reduce_scatter  # noqa: E402
 from pccl.build_kernels import build as build_pccl  # noqa: E402
 from benchmark_raw_collectives.utils import allclose, time_something, world_size_from_env  # noqa: E402
 
@@ -118,10 +119,16 @@ def main(argv=None):
                 for r in range(world_size):
                     assert allclose(outputs[r].float(), gold[r * output_numel:(r + 1) * output_numel], **tol)
 
-            # every rank adds (world-1) blocks: 2 reads + 1 write per element and hop
-            job_bytes = 3 * (world_size - 1) * output_numel * esize * world_size
+            # bytes the job moves: one fused pass reads every input once and writes every output; a
+            # per-step replay has every rank add (world-1) blocks, 2 reads + 1 write per element and hop
+            one_pass = args.library == "mpi" or (args.use_pccl_cpp_backend and
+                                                 kernels.mode_code(None) == kernels.MODE_FUSED)
+            if one_pass:
+                job_bytes = (world_size + 1) * world_size * output_numel * esize
+            else:
+                job_bytes = 3 * (world_size - 1) * output_numel * esize * world_size
             gbps = job_bytes / (time_ms * 1e-3) / 1e9
-            print(f"time_{library} = {time_ms:.3f} ms  ({gbps:.0f} GB/s algorithmic)")
+            print(f"time_{library} = {time_ms:.3f} ms  ({gbps:.0f} GB/s of bytes moved)")
             print("===============================")
             writer.writerow([gpu_count, slurm_job_id, size, unit, time_ms, job_bytes, round(gbps, 1),
                              round(100 * gbps / HBM_PEAK_GBPS, 2)])
