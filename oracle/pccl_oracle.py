@@ -33,8 +33,9 @@ holding the bfloat16 bit patterns.
 Pinning (see tests/test_oracle.py): the fp32 add is numpy's IEEE binary32 add;
 the bf16 add is checked against torch's CPU bfloat16 add over every exponent
 pair and against an independent integer rounding; the schedules are checked
-against closed-form summation orders (left fold from rank j+1, XOR butterfly),
-against exact integer sums, against P = 2 reducing to one add, against the C
+against closed-form summation orders (left fold from rank j+1, XOR butterfly;
+for the 2-D collectives the inner order inside every node, then the outer order
+across the nodes), against exact integer sums, against P = 2 reducing to one add, against the C
 restatement in pccl_oracle.c, and against the committed vectors in
 tests/golden/.  The reference ships no golden vectors of its own.
 """

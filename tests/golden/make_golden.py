@@ -8,7 +8,9 @@ are pinned independently by the closed forms in tests/test_oracle.py.  Each
 .npz holds the inputs of every rank and the expected output of every rank:
     in_<r>   rank r's input   (float32, or uint16 bfloat16 bit patterns)
     out_<r>  rank r's output
-    meta     JSON: collective, algorithm, dtype, P, block elements
+    meta     JSON: collective, algorithm, dtype, P, block elements; for the 2-D
+             collectives also the grid (intra, inter), for the uneven all_gather
+             the shard lengths and byte offsets
 Run:  python tests/golden/make_golden.py   (rewrites the files in place)
 """
 import json
@@ -46,7 +48,30 @@ CASES = [
     ("rs_halving_p2_f32", "reduce_scatter", "recursive", O.F32, 2, 64, "uniform"),
     ("ag_doubling_p8_bf16", "all_gather", "recursive", O.BF16, 8, 21, "normal"),
     ("ag_ring_p5_f32", "all_gather", "ring", O.F32, 5, 7, "normal"),
+    ("ar_halving_p4_f32", "all_reduce", "recursive", O.F32, 4, 13, "normal"),
+    ("ar_ring_p3_bf16", "all_reduce", "ring", O.BF16, 3, 11, "grad"),
 ]
+
+GRID_CASES = [
+    # name, collective, algorithm, dtype, intra, inter, elements per output block, input kind
+    ("rs2d_halving_2x2_bf16", "reduce_scatter_2d", "recursive", O.BF16, 2, 2, 17, "normal"),
+    ("rs2d_ring_3x2_f32", "reduce_scatter_2d", "ring", O.F32, 3, 2, 9, "uniform"),
+    ("rs2d_halving_4x2_f32", "reduce_scatter_2d", "recursive", O.F32, 4, 2, 5, "grad"),
+    ("ag2d_doubling_2x4_bf16", "all_gather_2d", "recursive", O.BF16, 2, 4, 6, "normal"),
+    ("ag2d_ring_3x2_f32", "all_gather_2d", "ring", O.F32, 3, 2, 10, "normal"),
+]
+
+UNEVEN_CASES = [
+    # name, shard lengths in bytes, gap between shards in bytes
+    ("ag_uneven_p5", [37, 0, 4096, 1, 513], 3),
+    ("ag_uneven_p3_packed", [100, 7, 64], 0),
+]
+
+
+def save(name, arrays, meta):
+    arrays["meta"] = np.frombuffer(json.dumps(meta).encode(), dtype=np.uint8)
+    np.savez(os.path.join(HERE, name + ".npz"), **arrays)
+    print("wrote", name)
 
 
 def main():
@@ -55,6 +80,9 @@ def main():
             xs = inputs(P, P * B, dtype, 1234, kind)
             fn = O.ring_reduce_scatter if alg == "ring" else O.recursive_halving_reduce_scatter
             outs = fn(xs, dtype)
+        elif coll == "all_reduce":
+            xs = inputs(P, P * B, dtype, 1234, kind)
+            outs = O.all_reduce(xs, dtype, alg)
         else:
             xs = inputs(P, B, dtype, 1234, kind)
             fn = O.ring_all_gather if alg == "ring" else O.recursive_doubling_all_gather
@@ -62,9 +90,29 @@ def main():
         arrays = {f"in_{r}": xs[r] for r in range(P)}
         arrays.update({f"out_{r}": outs[r] for r in range(P)})
         meta = dict(collective=coll, algorithm=alg, dtype=dtype, P=P, B=B, inputs=kind)
-        arrays["meta"] = np.frombuffer(json.dumps(meta).encode(), dtype=np.uint8)
-        np.savez(os.path.join(HERE, name + ".npz"), **arrays)
-        print("wrote", name)
+        save(name, arrays, meta)
+    for name, coll, alg, dtype, intra, inter, m, kind in GRID_CASES:
+        W = intra * inter
+        if coll == "reduce_scatter_2d":
+            xs = inputs(W, W * m, dtype, 4321, kind)
+            outs = O.reduce_scatter_2d(xs, intra, inter, dtype, alg)
+        else:
+            xs = inputs(W, m, dtype, 4321, kind)
+            outs = [o.view(xs[0].dtype) for o in O.all_gather_2d(xs, intra, inter, alg)]
+        arrays = {f"in_{r}": xs[r] for r in range(W)}
+        arrays.update({f"out_{r}": outs[r] for r in range(W)})
+        save(name, arrays, dict(collective=coll, algorithm=alg, dtype=dtype, P=W, B=m, intra=intra, inter=inter,
+                                inputs=kind))
+    for name, nbytes, gap in UNEVEN_CASES:
+        P = len(nbytes)
+        xs = [np.random.default_rng(99 + r).integers(0, 256, n, dtype=np.uint8) for r, n in enumerate(nbytes)]
+        off = [int(v) for v in np.cumsum([0] + [n + gap for n in nbytes[:-1]])]
+        total = off[-1] + nbytes[-1] + gap
+        outs = O.uneven_all_gather(xs, off, total)       # bytes outside the shards hold 0xA5
+        arrays = {f"in_{r}": xs[r] for r in range(P)}
+        arrays.update({f"out_{r}": outs[r] for r in range(P)})
+        save(name, arrays, dict(collective="all_gather_uneven", algorithm="ring", dtype="u8", P=P, nbytes=nbytes,
+                                dst_off=off, total=total, fill=0xA5))
 
 
 if __name__ == "__main__":

@@ -78,3 +78,36 @@ def halving_closed_form(inputs, dtype):
             T = [O.vector_add(T[k], T[k ^ d], dtype) for k in range(P)]
         outs.append(np.array(T[j], copy=True))
     return outs
+
+
+def _fold_in_schedule_order(xs, j, algorithm, dtype):
+    """What block j of a reduce_scatter over len(xs) ranks holds when rank k
+    contributed xs[k]: the ring's left fold from rank j+1, or the XOR butterfly."""
+    P = len(xs)
+    if algorithm == "ring":
+        acc = xs[(j + 1) % P]
+        for t in range(2, P + 1):
+            acc = O.vector_add(acc, xs[(j + t) % P], dtype)
+        return np.array(acc, copy=True)
+    T = list(xs)
+    for t in range(P.bit_length() - 1):
+        d = P >> (t + 1)
+        T = [O.vector_add(T[k], T[k ^ d], dtype) for k in range(P)]
+    return np.array(T[j], copy=True)
+
+
+def grid_closed_form(inputs, intra, inter, dtype, algorithm):
+    """reduce_scatter_2D in closed form: world rank w = node * intra + local ends
+    with block w of the total, summed first over the locals of every node in the
+    inner schedule's order for block `local`, then over the nodes in the outer
+    schedule's order for block `node`."""
+    W = intra * inter
+    m = inputs[0].size // W
+    outs = []
+    for w in range(W):
+        node, local = divmod(w, intra)
+        per_node = [_fold_in_schedule_order([inputs[n * intra + l][w * m:(w + 1) * m] for l in range(intra)],
+                                            local, algorithm, dtype) for n in range(inter)]
+        outs.append(_fold_in_schedule_order(per_node, node, algorithm, dtype))
+    return outs
+

@@ -235,18 +235,39 @@ def _golden_cases():
 
 @pytest.mark.parametrize("path", _golden_cases(), ids=lambda p: p.split("/")[-1][:-4])
 @pytest.mark.parametrize("mode", MODES)
-def test_golden_vectors(target, path, mode):
+def test_golden_vectors(target, path, mode, monkeypatch):
     """The committed fixtures (tests/golden/make_golden.py) through the library."""
     import json
     import torch
     from pccl import kernels
     z = np.load(path)
     meta = json.loads(bytes(z["meta"]).decode())
-    P, dtype = meta["P"], meta["dtype"]
+    P, dtype, kind = meta["P"], meta["dtype"], meta["collective"]
+    if kind == "all_gather_uneven":
+        t_in = [torch.from_numpy(z[f"in_{r}"].copy()).to(target.device) for r in range(P)]
+        t_out = [torch.full((meta["total"],), meta["fill"], dtype=torch.uint8, device=target.device) for _ in range(P)]
+        kernels.all_gather_uneven_ranks(t_out, t_in, meta["dst_off"])
+        target.sync()
+        for r in range(P):
+            assert np.array_equal(t_out[r].cpu().numpy(), z[f"out_{r}"]), f"rank {r}"
+        return
     t_in = [to_torch(z[f"in_{r}"], dtype, target.device) for r in range(P)]
-    if meta["collective"] == "reduce_scatter":
+    if kind == "all_reduce":
+        import pccl
+        world = pccl.VirtualWorld(P, target.device)
+        monkeypatch.setenv("PCCL_VIRTUAL_MODE", mode)
+        world.run(lambda comm: pccl._all_reduce(t_in[comm.Get_rank()], group=comm,
+                                                use_rh_and_rd=meta["algorithm"] == "recursive"))
+        t_out = t_in                                       # in place, like the reference
+    elif kind == "reduce_scatter":
         t_out = [torch.zeros(meta["B"], dtype=_tdtype(dtype), device=target.device) for _ in range(P)]
         kernels.reduce_scatter_ranks(t_out, t_in, meta["algorithm"], mode)
+    elif kind == "reduce_scatter_2d":
+        t_out = [torch.zeros(meta["B"], dtype=_tdtype(dtype), device=target.device) for _ in range(P)]
+        kernels.reduce_scatter_2d_ranks(t_out, t_in, meta["intra"], meta["inter"], meta["algorithm"], mode)
+    elif kind == "all_gather_2d":
+        t_out = [torch.zeros(P * meta["B"], dtype=_tdtype(dtype), device=target.device) for _ in range(P)]
+        kernels.all_gather_2d_ranks(t_out, t_in, meta["intra"], meta["inter"], meta["algorithm"], mode)
     else:
         t_out = [torch.zeros(P * meta["B"], dtype=_tdtype(dtype), device=target.device) for _ in range(P)]
         kernels.all_gather_ranks(t_out, t_in, meta["algorithm"], mode)

@@ -13,7 +13,7 @@ import subprocess
 import numpy as np
 import pytest
 
-from helpers import assert_bits_equal, halving_closed_form, make_inputs, ring_closed_form
+from helpers import assert_bits_equal, grid_closed_form, halving_closed_form, make_inputs, ring_closed_form
 from oracle import pccl_oracle as O
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -258,6 +258,31 @@ def test_reduce_scatter_2d_gives_block_r_of_the_total(alg, intra, inter):
         assert np.array_equal(outs[r], total[r * m:(r + 1) * m]), r
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("alg,intra,inter", [("ring", 2, 2), ("ring", 3, 2), ("ring", 4, 3), ("ring", 1, 5), ("ring", 5, 1),
+                                             ("recursive", 2, 2), ("recursive", 4, 2), ("recursive", 2, 8),
+                                             ("recursive", 8, 4)])
+def test_reduce_scatter_2d_rounds_in_the_order_of_both_levels(dtype, alg, intra, inter):
+    """Floating-point inputs: the bits fix the order of summation, first inside
+    every node, then across the nodes, each in its schedule's order."""
+    world = intra * inter
+    ins = make_inputs(world, world * 13, dtype, seed=14)
+    got = O.reduce_scatter_2d(ins, intra, inter, dtype, alg)
+    want = grid_closed_form(ins, intra, inter, dtype, alg)
+    for r in range(world):
+        assert_bits_equal(got[r], want[r], f"rank {r}")
+
+
+def test_2d_order_differs_from_the_flat_order_so_the_closed_form_has_teeth():
+    world, m = 8, 4096
+    ins = make_inputs(world, world * m, O.F32, seed=15)
+    grid = grid_closed_form(ins, 4, 2, O.F32, "ring")
+    flat = ring_closed_form(ins, O.F32)
+    swapped = grid_closed_form(ins, 2, 4, O.F32, "ring")
+    assert sum(int((a.view(np.uint32) != b.view(np.uint32)).sum()) for a, b in zip(grid, flat)) > 0
+    assert sum(int((a.view(np.uint32) != b.view(np.uint32)).sum()) for a, b in zip(grid, swapped)) > 0
+
+
 @pytest.mark.parametrize("alg", ["ring", "recursive"])
 @pytest.mark.parametrize("intra,inter", [(2, 2), (4, 2), (2, 4)])
 def test_all_gather_2d_is_concatenation_in_world_order(alg, intra, inter):
@@ -373,6 +398,30 @@ def test_oracle_reproduces_golden_vectors(path):
     meta = json.loads(bytes(z["meta"]).decode())
     P, dtype = meta["P"], meta["dtype"]
     ins = [z[f"in_{r}"] for r in range(P)]
+    kind = meta["collective"]
+    if kind in ("reduce_scatter_2d", "all_gather_2d", "all_reduce", "all_gather_uneven"):
+        # what the mathematics fixes first, then the oracle against the fixture
+        alg = meta["algorithm"]
+        if kind == "reduce_scatter_2d":
+            closed = grid_closed_form(ins, meta["intra"], meta["inter"], dtype, alg)
+            outs = O.reduce_scatter_2d(ins, meta["intra"], meta["inter"], dtype, alg)
+        elif kind == "all_gather_2d":
+            closed = [np.concatenate(ins)] * P
+            outs = [o.view(ins[0].dtype) for o in O.all_gather_2d(ins, meta["intra"], meta["inter"], alg)]
+        elif kind == "all_reduce":
+            blocks = (ring_closed_form if alg == "ring" else halving_closed_form)(ins, dtype)
+            closed = [np.concatenate(blocks)] * P
+            outs = O.all_reduce(ins, dtype, alg)
+        else:
+            one = np.full(meta["total"], meta["fill"], np.uint8)
+            for k in range(P):
+                one[meta["dst_off"][k]:meta["dst_off"][k] + meta["nbytes"][k]] = ins[k]
+            closed = [one] * P
+            outs = O.uneven_all_gather(ins, meta["dst_off"], meta["total"], meta["fill"])
+        for r in range(P):
+            assert_bits_equal(z[f"out_{r}"], closed[r], f"fixture vs closed form, rank {r}")
+            assert_bits_equal(outs[r], z[f"out_{r}"], f"oracle vs fixture, rank {r}")
+        return
     if meta["collective"] == "reduce_scatter":
         fn = O.ring_reduce_scatter if meta["algorithm"] == "ring" else O.recursive_halving_reduce_scatter
         outs = fn(ins, dtype)
