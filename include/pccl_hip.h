@@ -323,8 +323,8 @@ int pccl_hip_probe_mix(const void* const* reads, int nr, void* const* writes,
  *                  the Infinity Cache and the L2s, 288 MiB),
  *      "lds_pad" / "lds_pad_copy" / "lds_pad_kway" / "lds_pad_gather" (bytes of
  *                  unused LDS per workgroup, 0..65536: bounds the workgroups
- *                  resident per CU; -1, the default of lds_pad_kway and
- *                  lds_pad_gather, lets the launch choose),
+ *                  resident per CU; -1, the default of all but lds_pad,
+ *                  lets the launch choose),
  *      "unroll_gather" (vectors per thread of the all_gather placement kernels:
  *                  1, 2, 4, 8; 0, the default: one in the multicast kernel,
  *                  four in the time-blocked one),

@@ -53,7 +53,7 @@ std::atomic<long> g_unroll_copy{2};   // ... copy kernels (two 4 KiB chunks per 
 // share a CU (160 KiB of LDS): the fewer are resident, the narrower the address
 // window the chip streams from at any moment.  0 = as many as fit (8).
 std::atomic<long> g_lds_pad{0};        // add kernels
-std::atomic<long> g_lds_pad_copy{0};   // copy kernels
+std::atomic<long> g_lds_pad_copy{-1};  // copy kernels; -1 = chosen per launch (see copy_lds_pad)
 std::atomic<long> g_lds_pad_kway{-1};  // fused reduce; -1 = chosen per launch (see launch_kway)
 std::atomic<long> g_lds_pad_gather{-1}; // all_gather placement kernels; -1 = chosen per launch
 std::atomic<long> g_gather_split{0};   // groups of outputs per shard tile in the multicast gather; 0 = four outputs a group
@@ -257,15 +257,25 @@ int launch_add(const AddSegs& segs, int count, size_t n, int dtype, hipStream_t 
   return launch_add_pieces(segs, count, contiguous(n), dtype, stream, what);
 }
 
+// Unused LDS per workgroup of the copy kernels: six resident workgroups per CU
+// instead of eight for copies that stream from HBM (+1-1.5 % on MI355X from
+// 256 MiB per launch up); cache-sized copies keep all eight.
+unsigned copy_lds_pad(size_t traffic) {
+  const long pad = g_lds_pad_copy.load(std::memory_order_relaxed);
+  if (pad >= 0) return (unsigned)pad;
+  return stream_hint(-1, traffic) ? 24576u : 0u;
+}
+
 struct CopyLaunch {
   const CopySegs* segs;
   int count;
   size_t tiles;
   int aligned;
+  size_t traffic;
   hipStream_t stream;
   template <int U, bool NTL, bool NTS>
   void operator()() const {
-    const unsigned lds = (unsigned)g_lds_pad_copy.load();
+    const unsigned lds = copy_lds_pad(traffic);
     for_spans((size_t)count * tiles, 2 * kTileBytes * U, 1, 0, [&](Span span, unsigned grid) {
       hipLaunchKernelGGL((k_copy_segs<U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *segs, count, tiles, aligned, span);
     });
@@ -283,7 +293,7 @@ int launch_copy(const CopySegs& segs, int count, hipStream_t stream, const char*
   bool aligned = true;
   for (int s = 0; s < count && aligned; ++s)
     aligned = segs.nbytes[s] == 0 || (is16(segs.dst[s]) && is16(segs.src[s]) && (segs.nbytes[s] & 15u) == 0);
-  CopyLaunch l{&segs, count, copy_tiles_for(longest, t.unroll), aligned ? 1 : 0, stream};
+  CopyLaunch l{&segs, count, copy_tiles_for(longest, t.unroll), aligned ? 1 : 0, 2 * total, stream};
   if (int rc = check_work_items((size_t)count, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);
@@ -298,7 +308,7 @@ struct CopyPiecesLaunch {
   hipStream_t stream;
   template <int U, bool NTL, bool NTS>
   void operator()() const {
-    const unsigned lds = (unsigned)g_lds_pad_copy.load();
+    const unsigned lds = copy_lds_pad(2 * (size_t)count * pc.s1 * pc.s2 * pc.len);
     for_spans((size_t)count * pc.s1 * pc.s2 * tiles, 2 * kTileBytes * U, 1, 0, [&](Span span, unsigned grid) {
       hipLaunchKernelGGL((k_copy_pieces<U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *segs, count, pc, tiles, aligned, span);
     });
@@ -387,9 +397,11 @@ struct KwayLaunch {
     static_assert(U == 1, "the fused reduce is launched with one vector per thread");
 #define PCCL_KWAY(KV) \
   hipLaunchKernelGGL((k_reduce_kway<Acc, KV, U, NTL, NTS>), dim3(grid), dim3(kThreads), lds_pad, stream, *args, k, g, nout, n, first0, tiles, span)
-    // folds over at most 16 shards go out as launches 1.5 times the size of the add kernels' (+2 %);
-    // longer folds lose more to the drain of a launch than they gain, and stay one launch
-    for_spans((size_t)nout * tiles, kTileBytes * U * ((size_t)k + 1), 1, k <= 16 ? add_launch_mib() * 3 / 2 : 0, [&](Span span, unsigned grid) {
+    // folds over at most 16 shards go out as launches 1.5 times (butterfly order, +2-4 %) or 3 times
+    // (ring order, +1-2 %) the size of the add kernels'; longer folds lose more to the drain of a
+    // launch than they gain, and stay one launch
+    const long span_mib = k > 16 ? 0 : order == PCCL_HIP_ORDER_RING ? add_launch_mib() * 3 : add_launch_mib() * 3 / 2;
+    for_spans((size_t)nout * tiles, kTileBytes * U * ((size_t)k + 1), 1, span_mib, [&](Span span, unsigned grid) {
       if (order == PCCL_HIP_ORDER_RING) { PCCL_KWAY(0); return; }
       switch (k) {
         case 2: PCCL_KWAY(2); break;
@@ -412,23 +424,43 @@ struct KwayLaunch {
   }
 };
 
+// Unused LDS per workgroup of the fused reduce, chosen for a launch.  It takes
+// the room of further workgroups on a CU (160 KiB of LDS: 21 KiB leave 7
+// resident, 24 KiB 6, 30 KiB 5, 32 KiB 4, 48 KiB 3; 8 without), and fewer
+// resident workgroups narrow the window each of the k streams has in flight.
+// Measured on MI355X on 4 GiB of operands, against 8 per CU, operands carved
+// from one allocation and allocated one by one alike:
+//   ring order, bf16:   3-15 shards 7 per CU +2-5 % (6 is as good or better for
+//                       8 and more shards in some placements of the operands'
+//                       pages and 2 % worse in others), 16 and more 4 +5-8 %;
+//   ring order, fp32:   5-15 shards 6 +1-4 %, 16-23 shards 4 +6-8 %, 24 and more
+//                       3 +7-14 % (4 below 768 MiB of traffic);
+//   two-level ring:     bf16 7 (up to 8 shards) or 6, +2-4 %; fp32 5, +4-8 %;
+//   halving butterfly:  fp32 8 and 16 shards 4 per CU, +2-7 %; its other sizes
+//                       and bf16 gain in one placement what they lose in another.
+// All of it holds for streams from HBM only: operands that fit the caches (up
+// to about 256 MiB of traffic) lose 2-9 % with fewer workgroups, so the
+// footprint rule of the non-temporal hints decides here too.
+long kway_lds_pad(int k, int g, int dtype, int order, size_t traffic) {
+  if (!stream_hint(-1, traffic)) return 0;
+  const bool f32 = dtype == PCCL_HIP_F32;
+  if (order == PCCL_HIP_ORDER_RING) {
+    if (g >= k) {
+      if (f32) return k >= 24 ? (traffic >= ((size_t)768 << 20) ? 49152 : 32768) : k >= 16 ? 32768 : k >= 5 ? 24576 : 0;
+      return k >= 16 ? 32768 : k >= 3 ? 21504 : 0;
+    }
+    if (f32) return 30720;
+    return k <= 8 ? 21504 : 24576;
+  }
+  return f32 && (k == 8 || k == 16) ? 32768 : 0;
+}
+
 // g = size of the inner groups of a two-level ring order (g >= k: one level).
 int launch_kway(const KwayArgs& args, int k, int g, int nout, size_t n, int dtype, int order,
                 int first0, int per_hop, hipStream_t stream, const char* what) {
   if (n == 0 || nout == 0) return PCCL_HIP_OK;
-  // Fewer resident workgroups per CU (unused LDS takes the room) narrow the
-  // window each of the k streams has in flight.  Measured on MI355X, 4 GiB read:
-  // five per CU (32 KiB each) for one-level ring folds over 16 or more shards,
-  // +3-5 %; six per CU (24 KiB) for fp32 folds over 8-15 shards, +7 %; bf16
-  // below 16 shards, folds over fewer than 8 and the butterfly order lose from it.
   long pad = g_lds_pad_kway.load(std::memory_order_relaxed);
-  if (pad < 0) {
-    pad = 0;
-    if (order == PCCL_HIP_ORDER_RING && g >= k) {
-      if (k >= 16) pad = 32768;
-      else if (k >= 8 && dtype == PCCL_HIP_F32) pad = 24576;
-    }
-  }
+  if (pad < 0) pad = kway_lds_pad(k, g, dtype, order, ((size_t)k + 1) * n * esize_of(dtype) * (size_t)nout);
   KwayLaunch l{&args, k, g, nout, dtype, order, first0, per_hop, n, tiles_for(n * esize_of(dtype), 1),
                (unsigned)pad, stream};
   if (int rc = check_work_items((size_t)nout, l.tiles, what)) return rc;
@@ -527,7 +559,7 @@ int pccl_hip_set_tuning(const char* key, long value) {
       return fail(PCCL_HIP_EINVAL, "set_tuning: unroll_copy must be 1, 2, 4 or 8");
     g_unroll_copy = value;
   } else if (!strcmp(key, "lds_pad") || !strcmp(key, "lds_pad_copy") || !strcmp(key, "lds_pad_kway")) {
-    const long lowest = !strcmp(key, "lds_pad_kway") ? -1 : 0;   // -1: the fused reduce picks per launch
+    const long lowest = !strcmp(key, "lds_pad") ? 0 : -1;   // -1: the copies and the fused reduce pick per launch
     if (value < lowest || value > 65536)
       return fail(PCCL_HIP_EINVAL, "set_tuning: %s must be in [%ld, 65536]", key, lowest);
     (!strcmp(key, "lds_pad") ? g_lds_pad : !strcmp(key, "lds_pad_copy") ? g_lds_pad_copy : g_lds_pad_kway) = value;
