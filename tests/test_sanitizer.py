@@ -21,3 +21,20 @@ def test_kernels_stay_in_bounds_under_address_sanitizer():
                        capture_output=True, text=True, env=env, timeout=900)
     assert p.returncode == 0, (p.stdout[-2000:], p.stderr[-4000:])
     assert "ASAN CHECK OK" in p.stdout
+
+
+def test_kernels_show_no_undefined_behaviour():
+    """The same drive with UndefinedBehaviorSanitizer: misaligned vector accesses,
+    shifts and integer overflow in the index arithmetic would print a runtime error."""
+    runtimes = glob.glob("/opt/rocm/lib/llvm/lib/clang/*/lib/linux/libclang_rt.ubsan_standalone-x86_64.so")
+    if not os.path.exists(HOST_CLANG) or not runtimes:
+        pytest.skip("no host clang++ with a shared UndefinedBehaviorSanitizer runtime")
+    lib = build_cpu_library(out=EMUL_SO.replace(".so", "_ubsan.so"),
+                            extra_flags=("-fsanitize=undefined", "-fno-sanitize=vptr", "-shared-libsan",
+                                         "-fno-omit-frame-pointer"))
+    env = dict(os.environ, LD_PRELOAD=runtimes[0], UBSAN_OPTIONS="print_stacktrace=1:halt_on_error=0")
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "asan_check.py"), lib],
+                       capture_output=True, text=True, env=env, timeout=900)
+    assert p.returncode == 0, (p.stdout[-2000:], p.stderr[-4000:])
+    assert "runtime error" not in p.stderr, p.stderr[-4000:]
+    assert "ASAN CHECK OK" in p.stdout
