@@ -269,3 +269,62 @@ def test_indexing_beyond_4gib():
     # the tail window [2^31 - 37655, 2^31 + 12345) straddles byte offset 2^32
     want = O.vector_add(to_numpy(tail, O.BF16), np.full(50000, 0x4000, np.uint16), O.BF16)
     assert_bits_equal(to_numpy(a[-50000:], O.BF16), want, "window across the 4 GiB line")
+
+
+@pytest.mark.parametrize("alg,P,dtype", [("ring", 4, O.BF16), ("ring", 16, O.BF16), ("ring", 6, O.F32), ("ring", 16, O.F32),
+                                         ("ring", 24, O.F32), ("recursive", 8, O.F32), ("recursive", 16, O.F32),
+                                         ("recursive", 8, O.BF16)])
+def test_fused_reduce_at_streaming_sizes_equals_the_steps(alg, P, dtype):
+    """From 288 MiB of traffic on the fused reduce runs with fewer workgroups per
+    CU, a number chosen by shard count, element type and order: every such choice
+    gives the bits of the per-step replay, and exact totals on integer inputs."""
+    import torch
+    from pccl import kernels
+    es = 4 if dtype == O.F32 else 2
+    td = torch.float32 if dtype == O.F32 else torch.bfloat16
+    B = (1024 * MiB // es // P // P) // 128 * 128 + 8          # about 1 GiB of inputs, blocks not a multiple of a tile
+    ins = [_gen(P * B, dtype, 900 + r, kind="int") for r in range(P)]
+    total = torch.zeros(P * B, device=DEV)
+    for t in ins:
+        total += t.float()
+    outs = {}
+    for mode in ("steps", "fused"):
+        print(f"{alg} P={P} {dtype} mode={mode}", flush=True)
+        outs[mode] = [torch.zeros(B, dtype=td, device=DEV) for _ in range(P)]
+        kernels.reduce_scatter_ranks(outs[mode], ins, alg, mode)
+        torch.cuda.synchronize()
+    for r in range(P):
+        assert torch.equal(outs["fused"][r].float(), total[r * B:(r + 1) * B]), f"totals, rank {r}"
+        assert _same_bits(outs["fused"][r], outs["steps"][r]), f"rank {r}"
+    del ins, total
+    ins = [_gen(P * B, dtype, 950 + r) for r in range(P)]
+    for mode in ("steps", "fused"):
+        kernels.reduce_scatter_ranks(outs[mode], ins, alg, mode)
+        torch.cuda.synchronize()
+    for r in range(P):
+        assert _same_bits(outs["fused"][r], outs["steps"][r]), f"random inputs, rank {r}"
+    _check_rs_windows(outs["fused"], ins, P, B, dtype, alg)
+
+
+@pytest.mark.parametrize("intra,inter,dtype", [(4, 2, O.F32), (4, 2, O.BF16), (4, 4, O.BF16)])
+def test_fused_two_level_reduce_at_streaming_sizes_equals_the_steps(intra, inter, dtype):
+    import torch
+    from pccl import kernels
+    W = intra * inter
+    es = 4 if dtype == O.F32 else 2
+    td = torch.float32 if dtype == O.F32 else torch.bfloat16
+    m = (1024 * MiB // es // W // W) // 128 * 128 + 8
+    ins = [_gen(W * m, dtype, 700 + r) for r in range(W)]
+    outs = {}
+    for mode in ("steps", "fused"):
+        print(f"2-D ring {intra}x{inter} {dtype} mode={mode}", flush=True)
+        outs[mode] = [torch.zeros(m, dtype=td, device=DEV) for _ in range(W)]
+        kernels.reduce_scatter_2d_ranks(outs[mode], ins, intra, inter, "ring", mode)
+        torch.cuda.synchronize()
+    for w in range(W):
+        assert _same_bits(outs["fused"][w], outs["steps"][w]), f"rank {w}"
+    s, n = m // 2 + 5, 2053
+    sub = [np.concatenate([to_numpy(ins[k][j * m + s:j * m + s + n], dtype) for j in range(W)]) for k in range(W)]
+    want = O.reduce_scatter_2d(sub, intra, inter, dtype, "ring")
+    for w in range(W):
+        assert_bits_equal(to_numpy(outs["fused"][w][s:s + n], dtype), want[w], f"window, rank {w}")
