@@ -151,6 +151,10 @@ def reduce_kway(out: torch.Tensor, shards: Sequence[torch.Tensor], order: str = 
 
     order 'ring': shards first, first+1, ... (mod k) as a left fold;
     order 'halving': the butterfly of recursive halving rooted at `first`."""
+    # a call on the same tensor objects replays the checked arguments of the first (see _PLANS below)
+    key = ("kway", order, first, bool(per_hop_round), id(out), *map(id, shards))
+    if shards and _plan_lookup(key, (out,), shards):
+        return
     check_device_tensor(out, "out")
     for s in shards:
         check_device_tensor(s, "shard")
@@ -159,8 +163,14 @@ def reduce_kway(out: torch.Tensor, shards: Sequence[torch.Tensor], order: str = 
     code = {"ring": ORDER_RING, "halving": ORDER_HALVING}.get(order)
     if code is None:
         raise ValueError(f"unknown order {order!r}")
-    _native.load().reduce_kway(out.data_ptr(), _ptrs(shards), out.numel(), dtype_code(out.dtype), code,
-                               first, per_hop_round, stream_handle())
+    lib = _native.load()
+    table = _native._ptr_table(_ptrs(shards))
+    args = (out.data_ptr(), table, len(shards), out.numel(), dtype_code(out.dtype), code, first,
+            1 if per_hop_round else 0)
+    fn = lib._lib.pccl_hip_reduce_kway
+    if fn(*args, stream_handle()):
+        raise _native.NativeError(lib.last_error())
+    _plan_store(key, lib, fn, args, (table,), (out,), shards)
 
 
 def block_transpose(dst: torch.Tensor, src: torch.Tensor, rows: int, cols: int):

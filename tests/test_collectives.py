@@ -526,6 +526,47 @@ def test_repeated_calls_replay_the_checked_arguments(target, mode):
     assert not (set(kernels._PLANS) & mine)           # entries die with their tensors
 
 
+def test_repeated_folds_replay_the_checked_arguments(target):
+    """kernels.reduce_kway on the same tensor objects: fresh data, another order,
+    a storage swapped under a shard, a shard of another size."""
+    import gc
+    import torch
+    from pccl import kernels
+    k, n, dtype = 5, 1031, O.BF16
+    shards = [torch.zeros(n, dtype=torch.bfloat16, device=target.device) for _ in range(k)]
+    out = torch.zeros(n, dtype=torch.bfloat16, device=target.device)
+    gc.collect()
+    before = set(kernels._PLANS)
+
+    def want(xs, first):
+        acc = xs[first]
+        for t in range(1, k):
+            acc = O.vector_add(acc, xs[(first + t) % k], dtype)
+        return acc
+
+    for seed, first in ((61, 0), (62, 0), (63, 3), (64, 3)):
+        xs = make_inputs(k, n, dtype, seed=seed)
+        for t, x in zip(shards, xs):
+            t.copy_(to_torch(x, dtype, target.device))
+        kernels.reduce_kway(out, shards, "ring", first)
+        target.sync()
+        assert_bits_equal(to_numpy(out, dtype), want(xs, first), f"seed {seed}")
+    mine = set(kernels._PLANS) - before
+    assert len(mine) == 2                              # one entry per (tensors, order, first)
+    moved = to_torch(make_inputs(1, n, dtype, seed=65)[0], dtype, target.device)
+    shards[1].set_(moved.untyped_storage(), 0, moved.shape)
+    kernels.reduce_kway(out, shards, "ring", 3)
+    target.sync()
+    xs[1] = to_numpy(moved, dtype)
+    assert_bits_equal(to_numpy(out, dtype), want(xs, 3), "after set_")
+    shards[0].set_(torch.zeros(n + 1, dtype=torch.bfloat16, device=target.device).untyped_storage(), 0, (n + 1,))
+    with pytest.raises(RuntimeError, match="shards must match"):
+        kernels.reduce_kway(out, shards, "ring", 3)
+    del shards, out, moved
+    gc.collect()
+    assert not (set(kernels._PLANS) & mine)
+
+
 @pytest.mark.parametrize("rec,kwargs", [(True, {}), (False, {}), (True, {"use_yacl": True}),
                                         (False, {"use_yacl": True, "use_pccl_cpp_backend": False}),
                                         (False, {"directly_call_mpi": True})])
