@@ -847,7 +847,7 @@ def cpu_baseline(info):
 
 # ---------------------------------------------------------------------------
 
-TUNING_KEYS = ("grid_cap", "unroll", "unroll_copy", "nt_load", "nt_store", "launch_mib", "gather_strip",
+TUNING_KEYS = ("grid_cap", "unroll", "add_rows", "launch_mib_rows", "unroll_copy", "nt_load", "nt_store", "launch_mib", "gather_strip",
                "gather_split", "unroll_gather", "gather_nt", "lds_pad", "lds_pad_copy", "lds_pad_kway",
                "lds_pad_gather")
 

@@ -47,7 +47,10 @@ int launch_status(const char* what) {
 }
 
 std::atomic<long> g_grid_cap{0};
-std::atomic<long> g_unroll{4};        // vectors per thread and operand, add kernels
+std::atomic<long> g_unroll{4};        // vectors per thread and operand, general add kernels
+// Aligned contiguous adds go to the lean one-wave kernels (k_add_rows, k_rh_rows); 0 = always the general kernels
+std::atomic<long> g_add_rows{1};
+std::atomic<long> g_launch_mib_rows{0};   // traffic per launch of the lean add kernels, MiB (0 = a step is one launch)
 std::atomic<long> g_unroll_copy{2};   // ... copy kernels (two 4 KiB chunks per workgroup, 8 chunks apart: see copy_vec)
 // Unused dynamic LDS requested per workgroup, only to bound how many workgroups
 // share a CU (160 KiB of LDS): the fewer are resident, the narrower the address
@@ -148,10 +151,10 @@ void for_spans(size_t items, size_t item_bytes, size_t multiple, long target_mib
 
 long add_launch_mib() { return g_launch_mib.load(std::memory_order_relaxed); }
 
-size_t tiles_for(size_t nbytes, int unroll) {
+size_t tiles_for(size_t nbytes, int unroll, int threads = kThreads) {
   // one extra vector covers the shift of the body behind an unaligned head
   size_t nvec = nbytes / 16 + 2;
-  size_t per = (size_t)kThreads * (size_t)unroll;
+  size_t per = (size_t)threads * (size_t)unroll;
   return (nvec + per - 1) / per;
 }
 
@@ -164,6 +167,7 @@ size_t copy_tiles_for(size_t nbytes, int unroll) {
 struct Tune {
   int unroll;
   bool ntl, nts;
+  int threads;   // workgroup size of the add kernels
 };
 
 bool is16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
@@ -173,6 +177,7 @@ bool is16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 Tune current_tune(bool copy, size_t launch_bytes) {
   Tune t;
   t.unroll = (int)(copy ? g_unroll_copy : g_unroll).load(std::memory_order_relaxed);
+  t.threads = kThreads;
   t.ntl = stream_hint(g_nt_load.load(std::memory_order_relaxed), launch_bytes);
   t.nts = stream_hint(g_nt_store.load(std::memory_order_relaxed), launch_bytes);
   return t;
@@ -217,19 +222,74 @@ struct AddLaunch {
   int count, dtype;
   Pieces pc;
   size_t tiles;
-  int aligned;
+  int aligned, threads;
   hipStream_t stream;
-  template <int U, bool NTL, bool NTS>
-  void operator()() const {
+  template <int U, bool NTL, bool NTS, int T>
+  void run() const {
     const unsigned lds = (unsigned)g_lds_pad.load();
-    for_spans((size_t)count * pc.s1 * pc.s2 * tiles, 3 * kTileBytes * U, 1, add_launch_mib(), [&](Span span, unsigned grid) {
+    for_spans((size_t)count * pc.s1 * pc.s2 * tiles, (size_t)3 * T * 16 * U, 1, add_launch_mib(), [&](Span span, unsigned grid) {
       if (dtype == PCCL_HIP_F32)
-        hipLaunchKernelGGL((k_add_segs<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *segs, count, pc, tiles, aligned, span);
+        hipLaunchKernelGGL((k_add_segs<OpF32, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *segs, count, pc, tiles, aligned, span);
       else
-        hipLaunchKernelGGL((k_add_segs<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *segs, count, pc, tiles, aligned, span);
+        hipLaunchKernelGGL((k_add_segs<OpBF16, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *segs, count, pc, tiles, aligned, span);
     });
   }
+  template <int U, bool NTL, bool NTS>
+  void operator()() const {
+    run<U, NTL, NTS, kThreads>();
+  }
 };
+
+// Calls launch(row0, nrows, tile0, ntiles) for the launches of a lean add step:
+// `rows` segments of `tiles` one-vector-per-thread tiles each, in pieces of
+// about target_mib MiB (0 = one launch) cut between rows where a piece holds
+// whole rows, inside a row otherwise.
+template <class F>
+void for_rows(int rows, size_t tiles, size_t tile_bytes, long target_mib, F&& launch) {
+  if (rows <= 0 || tiles == 0) return;
+  int rows_per = rows;
+  size_t tiles_per = tiles;
+  if (target_mib > 0) {
+    const double total = (double)rows * (double)tiles * (double)tile_bytes;
+    size_t pieces = (size_t)(total / ((double)target_mib * 1048576.0) + 0.5);
+    if (pieces < 1) pieces = 1;
+    if (pieces <= (size_t)rows) {
+      rows_per = (int)(((size_t)rows + pieces - 1) / pieces);
+    } else {
+      rows_per = 1;
+      const size_t per_row = (pieces + (size_t)rows - 1) / (size_t)rows;
+      tiles_per = (tiles + per_row - 1) / per_row;
+    }
+  }
+  if (rows_per > 65535) rows_per = 65535;
+  if (tiles_per > kMaxGrid) tiles_per = kMaxGrid;
+  for (int r0 = 0; r0 < rows; r0 += rows_per) {
+    const int nr = rows - r0 < rows_per ? rows - r0 : rows_per;
+    for (size_t t0 = 0; t0 < tiles; t0 += tiles_per) {
+      const size_t nt = tiles - t0 < tiles_per ? tiles - t0 : tiles_per;
+      launch(r0, nr, (uint32_t)t0, (unsigned)nt);
+      g_launches.fetch_add(1, std::memory_order_relaxed);
+    }
+  }
+}
+
+// The lean add for `count` contiguous, aligned segments of n elements.
+void launch_add_rows(const AddSegs& segs, int count, size_t n, int dtype, const Tune& t, hipStream_t stream) {
+  const size_t nvec = n * esize_of(dtype) / 16;
+  const size_t tiles = (nvec + kRowThreads - 1) / kRowThreads;
+  for_rows(count, tiles, (size_t)3 * kRowThreads * 16, g_launch_mib_rows.load(std::memory_order_relaxed),
+           [&](int row0, int nrows, uint32_t tile0, unsigned ntiles) {
+#define PCCL_ROWS(OP, L, S) hipLaunchKernelGGL((k_add_rows<OP, L, S>), dim3(ntiles, (unsigned)nrows), dim3(kRowThreads), 0, stream, segs, row0, nvec, tile0)
+    if (dtype == PCCL_HIP_F32) {
+      if (t.ntl) { if (t.nts) PCCL_ROWS(OpF32, true, true); else PCCL_ROWS(OpF32, true, false); }
+      else { if (t.nts) PCCL_ROWS(OpF32, false, true); else PCCL_ROWS(OpF32, false, false); }
+    } else {
+      if (t.ntl) { if (t.nts) PCCL_ROWS(OpBF16, true, true); else PCCL_ROWS(OpBF16, true, false); }
+      else { if (t.nts) PCCL_ROWS(OpBF16, false, true); else PCCL_ROWS(OpBF16, false, false); }
+    }
+#undef PCCL_ROWS
+  });
+}
 
 // True if every piece of every operand starts on a 16-byte boundary and is a
 // whole number of vectors: the kernels then skip all head/tail handling.
@@ -246,7 +306,13 @@ int launch_add_pieces(const AddSegs& segs, int count, const Pieces& pc, int dtyp
   Tune t = current_tune(false, 3 * (size_t)count * pc.s1 * pc.s2 * pc.len * esize_of(dtype));
   bool aligned = pieces_aligned(pc, esize_of(dtype));
   for (int s = 0; s < count && aligned; ++s) aligned = is16(segs.dst[s]) && is16(segs.a[s]) && is16(segs.b[s]);
-  AddLaunch l{&segs, count, dtype, pc, tiles_for(pc.len * esize_of(dtype), t.unroll), aligned ? 1 : 0, stream};
+  if (aligned && pc.s1 == 1 && pc.s2 == 1 && g_add_rows.load(std::memory_order_relaxed) &&
+      pc.len * esize_of(dtype) / 16 <= kMaxWorkItems * (size_t)kRowThreads) {
+    launch_add_rows(segs, count, pc.len, dtype, t, stream);
+    return launch_status(what);
+  }
+  AddLaunch l{&segs, count, dtype, pc, tiles_for(pc.len * esize_of(dtype), t.unroll, t.threads), aligned ? 1 : 0,
+              t.threads, stream};
   if (int rc = check_work_items((size_t)count * pc.s1 * pc.s2, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);
@@ -333,17 +399,21 @@ struct RhLaunch {
   const RhArgs* args;
   int P, round, dtype, from_src, to_outs;
   size_t B, tiles;
-  int aligned;
+  int aligned, threads;
   hipStream_t stream;
+  template <int U, bool NTL, bool NTS, int T>
+  void run() const {
+    const unsigned lds = (unsigned)g_lds_pad.load();
+    for_spans((size_t)P * tiles, (size_t)3 * T * 16 * U, 1, add_launch_mib(), [&](Span span, unsigned grid) {
+      if (dtype == PCCL_HIP_F32)
+        hipLaunchKernelGGL((k_rh_round<OpF32, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *args, P, B, round, from_src, to_outs, tiles, aligned, span);
+      else
+        hipLaunchKernelGGL((k_rh_round<OpBF16, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *args, P, B, round, from_src, to_outs, tiles, aligned, span);
+    });
+  }
   template <int U, bool NTL, bool NTS>
   void operator()() const {
-    const unsigned lds = (unsigned)g_lds_pad.load();
-    for_spans((size_t)P * tiles, 3 * kTileBytes * U, 1, add_launch_mib(), [&](Span span, unsigned grid) {
-      if (dtype == PCCL_HIP_F32)
-        hipLaunchKernelGGL((k_rh_round<OpF32, U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *args, P, B, round, from_src, to_outs, tiles, aligned, span);
-      else
-        hipLaunchKernelGGL((k_rh_round<OpBF16, U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *args, P, B, round, from_src, to_outs, tiles, aligned, span);
-    });
+    run<U, NTL, NTS, kThreads>();
   }
 };
 
@@ -554,6 +624,11 @@ int pccl_hip_set_tuning(const char* key, long value) {
     if (value != 1 && value != 2 && value != 4 && value != 8)
       return fail(PCCL_HIP_EINVAL, "set_tuning: unroll must be 1, 2, 4 or 8");
     g_unroll = value;
+  } else if (!strcmp(key, "add_rows")) {
+    g_add_rows = value != 0;
+  } else if (!strcmp(key, "launch_mib_rows")) {
+    if (value < 0) return fail(PCCL_HIP_EINVAL, "set_tuning: launch_mib_rows must be >= 0");
+    g_launch_mib_rows = value;
   } else if (!strcmp(key, "unroll_copy")) {
     if (value != 1 && value != 2 && value != 4 && value != 8)
       return fail(PCCL_HIP_EINVAL, "set_tuning: unroll_copy must be 1, 2, 4 or 8");
@@ -597,6 +672,8 @@ long pccl_hip_get_tuning(const char* key) {
   if (!key) return -1;
   if (!strcmp(key, "grid_cap")) return g_grid_cap;
   if (!strcmp(key, "unroll")) return g_unroll;
+  if (!strcmp(key, "add_rows")) return g_add_rows;
+  if (!strcmp(key, "launch_mib_rows")) return g_launch_mib_rows;
   if (!strcmp(key, "unroll_copy")) return g_unroll_copy;
   if (!strcmp(key, "lds_pad")) return g_lds_pad;
   if (!strcmp(key, "lds_pad_copy")) return g_lds_pad_copy;
@@ -678,8 +755,29 @@ int pccl_hip_rh_round(void* const* bufs, const void* const* src, void* const* ou
   bool aligned = (B * esize_of(dtype)) % 16 == 0;
   for (int r = 0; r < P && aligned; ++r)
     aligned = is16(args.bufs[r]) && is16(args.src[r]) && is16(args.outs[r]);
+  if (aligned && g_add_rows.load(std::memory_order_relaxed) && count * esize_of(dtype) / 16 <= kMaxWorkItems * (size_t)kRowThreads) {
+    const size_t nvec = count * esize_of(dtype) / 16;
+    const size_t tiles = (nvec + kRowThreads - 1) / kRowThreads;
+    int log2_group = 0;
+    while ((1 << log2_group) < (P >> round)) ++log2_group;
+    const int from_src = src ? 1 : 0, outs_i = to_outs ? 1 : 0;
+    hipStream_t st = (hipStream_t)stream;
+    for_rows(P, tiles, (size_t)3 * kRowThreads * 16, g_launch_mib_rows.load(std::memory_order_relaxed),
+             [&](int row0, int nrows, uint32_t tile0, unsigned ntiles) {
+#define PCCL_RH(OP, L, S) hipLaunchKernelGGL((k_rh_rows<OP, L, S>), dim3(ntiles, (unsigned)nrows), dim3(kRowThreads), 0, st, args, row0, log2_group, B, from_src, outs_i, nvec, tile0)
+      if (dtype == PCCL_HIP_F32) {
+        if (t.ntl) { if (t.nts) PCCL_RH(OpF32, true, true); else PCCL_RH(OpF32, true, false); }
+        else { if (t.nts) PCCL_RH(OpF32, false, true); else PCCL_RH(OpF32, false, false); }
+      } else {
+        if (t.ntl) { if (t.nts) PCCL_RH(OpBF16, true, true); else PCCL_RH(OpBF16, true, false); }
+        else { if (t.nts) PCCL_RH(OpBF16, false, true); else PCCL_RH(OpBF16, false, false); }
+      }
+#undef PCCL_RH
+    });
+    return launch_status(what);
+  }
   RhLaunch l{&args, P, round, dtype, src ? 1 : 0, to_outs ? 1 : 0, B,
-             tiles_for(count * esize_of(dtype), t.unroll), aligned ? 1 : 0, (hipStream_t)stream};
+             tiles_for(count * esize_of(dtype), t.unroll, t.threads), aligned ? 1 : 0, t.threads, (hipStream_t)stream};
   if (int rc = check_work_items((size_t)P, l.tiles, what)) return rc;
   with_tuning(t, l);
   return launch_status(what);

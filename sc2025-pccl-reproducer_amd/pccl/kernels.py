@@ -198,16 +198,17 @@ def block_transpose(dst: torch.Tensor, src: torch.Tensor, rows: int, cols: int):
 # 16 us of host time through the checks against 4 us of GPU time).  An entry is
 # keyed by the identities of the tensors; it holds no reference to them and is
 # dropped when one of them dies, so an identity cannot come back as another
-# tensor while its entry exists.  A replay still compares every tensor's current
-# address with the recorded one (storage swapped under the same object) and the
-# first input's and output's length.  Calls whose work buffers come from the
-# allocator per call are not kept.
+# tensor while its entry exists.  A replay still compares what the C call
+# depends on for EVERY tensor of the call, work buffers included: its current
+# address (storage swapped under the same object by set_() or .data), its
+# length (resize_()), its element type and that it is still contiguous.  Calls
+# whose work buffers come from the allocator per call are not kept.
 _PLANS = {}
 _PLANS_MAX = 512
 
 
 class _Plan:
-    __slots__ = ("lib", "fn", "args", "ptrs", "lens", "tables", "finals", "__weakref__")
+    __slots__ = ("lib", "fn", "args", "state", "tables", "finals", "__weakref__")
 
 
 def _plan_drop(key):
@@ -217,13 +218,16 @@ def _plan_drop(key):
             f.detach()
 
 
-def _plan_lookup(key, tensors_a, tensors_b):
+def _plan_state(*groups):
+    """What a recorded argument pack depends on, per tensor of the call."""
+    return [(t.data_ptr(), t.numel(), t.dtype, t.is_contiguous()) for g in groups for t in g]
+
+
+def _plan_lookup(key, tensors_a, tensors_b, extra=()):
     ent = _PLANS.get(key)
     if ent is None:
         return False
-    if (ent.lib is _native._loaded
-            and ent.ptrs == (*[t.data_ptr() for t in tensors_a], *[t.data_ptr() for t in tensors_b])
-            and ent.lens == (tensors_a[0].numel(), tensors_b[0].numel())):
+    if ent.lib is _native._loaded and ent.state == _plan_state(tensors_a, tensors_b, extra):
         if ent.fn(*ent.args, stream_handle()):
             raise _native.NativeError(ent.lib.last_error())
         return True
@@ -238,8 +242,7 @@ def _plan_store(key, lib, fn, args, tables, tensors_a, tensors_b, extra=()):
             _plan_drop(k)
     ent = _Plan()
     ent.lib, ent.fn, ent.args, ent.tables = lib, fn, args, tables
-    ent.ptrs = (*[t.data_ptr() for t in tensors_a], *[t.data_ptr() for t in tensors_b])
-    ent.lens = (tensors_a[0].numel(), tensors_b[0].numel())
+    ent.state = _plan_state(tensors_a, tensors_b, extra)
     ent.finals = [weakref.finalize(t, _plan_drop, key) for t in (*tensors_a, *tensors_b, *extra)]
     _PLANS[key] = ent
 
@@ -256,8 +259,9 @@ def reduce_scatter_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[torch
     P = len(inputs)
     if len(outputs) != P or P < 1:
         raise ValueError("need one output per input rank")
-    key = ("rs", algorithm, mode, *map(id, outputs), *map(id, inputs), *(() if work is None else map(id, work)))
-    if _plan_lookup(key, outputs, inputs):
+    m = mode_code(mode)          # the resolved mode: None follows $PCCL_VIRTUAL_MODE as it is now
+    key = ("rs", algorithm, m, *map(id, outputs), *map(id, inputs), None, *(() if work is None else map(id, work)))
+    if _plan_lookup(key, outputs, inputs, () if work is None else work):
         return
     if P > MAX_VIRTUAL_RANKS:
         raise RuntimeError(f"at most {MAX_VIRTUAL_RANKS} virtual ranks per communicator")
@@ -278,7 +282,6 @@ def reduce_scatter_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[torch
             raise RuntimeError("Output tensor must have block_size elements (input tensor numel()/world_size)")
         if o.dtype != dt:
             raise RuntimeError("Output tensor must be of type float (same dtype as the input)")
-    m = mode_code(mode)
     need_work = _needs_work(m, P, algorithm)
     own_work = need_work and work is None
     if own_work:
@@ -295,9 +298,8 @@ def reduce_scatter_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[torch
     fn = lib._lib.pccl_hip_reduce_scatter_virtual
     if fn(*args, stream_handle()):
         raise _native.NativeError(lib.last_error())
-    # mode None follows the environment, which may change between calls: such calls are not kept
-    if not own_work and (mode is not None or "PCCL_VIRTUAL_MODE" not in os.environ):
-        _plan_store(key, lib, fn, args, tables, outputs, inputs, work if need_work else ())
+    if not own_work:
+        _plan_store(key, lib, fn, args, tables, outputs, inputs, () if work is None else work)
 
 
 def _needs_work(m: int, P: int, algorithm: str) -> bool:
@@ -363,7 +365,8 @@ def all_gather_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[torch.Ten
     P = len(inputs)
     if len(outputs) != P or P < 1:
         raise ValueError("need one output per input rank")
-    key = ("ag", algorithm, mode, *map(id, outputs), *map(id, inputs))
+    m = mode_code(mode)
+    key = ("ag", algorithm, m, *map(id, outputs), *map(id, inputs))
     if _plan_lookup(key, outputs, inputs):
         return
     if P > MAX_VIRTUAL_RANKS:
@@ -384,12 +387,11 @@ def all_gather_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[torch.Ten
             raise RuntimeError("Output tensor must have total_elem elements (input tensor numel() *world_size)")
     lib = _native.load()
     tables = (_native._ptr_table(_ptrs(outputs)), _native._ptr_table(_ptrs(inputs)))
-    args = (*tables, P, blk * inputs[0].element_size(), algorithm.encode(), mode_code(mode))
+    args = (*tables, P, blk * inputs[0].element_size(), algorithm.encode(), m)
     fn = lib._lib.pccl_hip_all_gather_virtual
     if fn(*args, stream_handle()):
         raise _native.NativeError(lib.last_error())
-    if mode is not None or "PCCL_VIRTUAL_MODE" not in os.environ:
-        _plan_store(key, lib, fn, args, tables, outputs, inputs)
+    _plan_store(key, lib, fn, args, tables, outputs, inputs)
 
 
 # Distance added between the buffers of successive virtual ranks when they are

@@ -2,7 +2,7 @@
 // library's unchanged source be compiled for the CPU so that every kernel's
 // indexing can be checked under AddressSanitizer and compared with the oracle
 // without a GPU.  A launch runs the kernel once per (workgroup, thread) in
-// sequence; that is exact for these kernels because they use no LDS, no
+// sequence (grids of one or two dimensions); that is exact for these kernels because they use no LDS, no
 // barriers and no cross-thread communication.  Never part of the product.
 #pragma once
 #include <cstdint>
@@ -41,10 +41,11 @@ inline float __uint_as_float(uint32_t u) { float f; std::memcpy(&f, &u, 4); retu
     (void)(stream);                                                      \
     gridDim = (grid);                                                    \
     blockDim = (block);                                                  \
-    for (unsigned bx_ = 0; bx_ < gridDim.x; ++bx_)                       \
-      for (unsigned tx_ = 0; tx_ < blockDim.x; ++tx_) {                  \
-        blockIdx = dim3(bx_);                                            \
-        threadIdx = dim3(tx_);                                           \
-        kernel(__VA_ARGS__);                                             \
-      }                                                                  \
+    for (unsigned by_ = 0; by_ < gridDim.y; ++by_)                       \
+      for (unsigned bx_ = 0; bx_ < gridDim.x; ++bx_)                     \
+        for (unsigned tx_ = 0; tx_ < blockDim.x; ++tx_) {                \
+          blockIdx = dim3(bx_, by_, 0);                                  \
+          threadIdx = dim3(tx_, 0, 0);                                   \
+          kernel(__VA_ARGS__);                                           \
+        }                                                                \
   } while (0)
