@@ -57,6 +57,7 @@ sys.path.insert(0, os.path.join(ROOT, "sc2025-pccl-reproducer_amd"))
 METRIC = "reduce/copy kernel HBM GB/s and % of MI355X peak at 64MB-2GB messages"
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
 MiB = 1 << 20
+WARM_MS = 60.0               # least duration of the untimed warm-up before a timed region, see time_steps
 
 WORKLOADS = ["cfg1", "cfg2", "cfg3", "cfg3full", "cfg4", "cfg4u", "cfg5"]
 # every (workload, mode) row of the default run besides the headline cfg2/steps
@@ -478,6 +479,14 @@ def time_steps(step, steps, warmup, lib):
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
+    # The device needs about 20 ms of continuous streaming before its rate settles (per-call times of a 0.75 ms
+    # fold from a cold start: 0.82, 0.79, ... 0.73 of peak after 5 ms, 0.80 after 12 ms, 0.82-0.83 from 20 ms
+    # on), so the untimed warm-up is at least `warmup` steps AND at least WARM_MS of device work.
+    t_warm = time.perf_counter()
+    while (time.perf_counter() - t_warm) * 1e3 < WARM_MS:
+        for _ in range(max(1, warmup)):
+            step()
+        torch.cuda.synchronize()
     stream = torch.cuda.current_stream()
     start = torch.cuda.Event(enable_timing=True)
     end = torch.cuda.Event(enable_timing=True)
@@ -847,7 +856,7 @@ def cpu_baseline(info):
 
 # ---------------------------------------------------------------------------
 
-TUNING_KEYS = ("grid_cap", "unroll", "add_rows", "launch_mib_rows", "unroll_copy", "nt_load", "nt_store", "launch_mib", "gather_strip",
+TUNING_KEYS = ("grid_cap", "unroll", "add_rows", "launch_mib_rows", "wg_kway", "unroll_copy", "nt_load", "nt_store", "launch_mib", "gather_strip",
                "gather_split", "unroll_gather", "gather_nt", "lds_pad", "lds_pad_copy", "lds_pad_kway",
                "lds_pad_gather")
 

@@ -58,6 +58,7 @@ std::atomic<long> g_unroll_copy{2};   // ... copy kernels (two 4 KiB chunks per 
 std::atomic<long> g_lds_pad{0};        // add kernels
 std::atomic<long> g_lds_pad_copy{-1};  // copy kernels; -1 = chosen per launch (see copy_lds_pad)
 std::atomic<long> g_lds_pad_kway{-1};  // fused reduce; -1 = chosen per launch (see launch_kway)
+std::atomic<long> g_wg_kway{-1};       // threads per workgroup of the fused reduce: 64, 256, or -1 = 64 for streams from HBM
 std::atomic<long> g_lds_pad_gather{-1}; // all_gather placement kernels; -1 = chosen per launch
 std::atomic<long> g_gather_split{0};   // groups of outputs per shard tile in the multicast gather; 0 = four outputs a group
 std::atomic<long> g_gather_nt{-1};     // non-temporal stores in the all_gather placement kernels (-1: by footprint, like nt_store)
@@ -460,18 +461,15 @@ struct KwayLaunch {
   int k, g, nout, dtype, order, first0, per_hop;
   size_t n, tiles;
   unsigned lds_pad;
+  int threads;
   hipStream_t stream;
 
-  template <class Acc, int U, bool NTL, bool NTS>
-  void run() const {
+  template <class Acc, int U, bool NTL, bool NTS, int T, int PF>
+  void run_wg(long span_mib) const {
     static_assert(U == 1, "the fused reduce is launched with one vector per thread");
 #define PCCL_KWAY(KV) \
-  hipLaunchKernelGGL((k_reduce_kway<Acc, KV, U, NTL, NTS>), dim3(grid), dim3(kThreads), lds_pad, stream, *args, k, g, nout, n, first0, tiles, span)
-    // folds over at most 16 shards go out as launches 1.5 times (butterfly order, +2-4 %) or 3 times
-    // (ring order, +1-2 %) the size of the add kernels'; longer folds lose more to the drain of a
-    // launch than they gain, and stay one launch
-    const long span_mib = k > 16 ? 0 : order == PCCL_HIP_ORDER_RING ? add_launch_mib() * 3 : add_launch_mib() * 3 / 2;
-    for_spans((size_t)nout * tiles, kTileBytes * U * ((size_t)k + 1), 1, span_mib, [&](Span span, unsigned grid) {
+  hipLaunchKernelGGL((k_reduce_kway<Acc, KV, U, NTL, NTS, T, PF>), dim3(grid), dim3(T), lds_pad, stream, *args, k, g, nout, n, first0, tiles, span)
+    for_spans((size_t)nout * tiles, (size_t)T * 16 * U * ((size_t)k + 1), 1, span_mib, [&](Span span, unsigned grid) {
       if (order == PCCL_HIP_ORDER_RING) { PCCL_KWAY(0); return; }
       switch (k) {
         case 2: PCCL_KWAY(2); break;
@@ -483,6 +481,19 @@ struct KwayLaunch {
       }
     });
 #undef PCCL_KWAY
+  }
+
+  template <class Acc, int U, bool NTL, bool NTS>
+  void run() const {
+    if constexpr (NTL && NTS) {
+      // streams from HBM: one-wave workgroups, ring-order loads in pairs whatever k, one launch
+      if (threads == kRowThreads) { run_wg<Acc, U, NTL, NTS, kRowThreads, 2>(0); return; }
+    }
+    // 256 threads: folds over at most 16 shards go out as launches 1.5 times (butterfly order, +2-4 %) or
+    // 3 times (ring order, +1-2 %) the size of the add kernels'; longer folds lose more to the drain of a
+    // launch than they gain, and stay one launch
+    const long span_mib = k > 16 ? 0 : order == PCCL_HIP_ORDER_RING ? add_launch_mib() * 3 : add_launch_mib() * 3 / 2;
+    run_wg<Acc, U, NTL, NTS, kThreads, kFoldPairedFrom>(span_mib);
   }
 
   template <int U, bool NTL, bool NTS>
@@ -511,9 +522,20 @@ struct KwayLaunch {
 // All of it holds for streams from HBM only: operands that fit the caches (up
 // to about 256 MiB of traffic) lose 2-9 % with fewer workgroups, so the
 // footprint rule of the non-temporal hints decides here too.
-long kway_lds_pad(int k, int g, int dtype, int order, size_t traffic) {
+long kway_lds_pad(int k, int g, int dtype, int order, size_t traffic, int threads) {
   if (!stream_hint(-1, traffic)) return 0;
   const bool f32 = dtype == PCCL_HIP_F32;
+  if (threads == kRowThreads) {
+    // One-wave workgroups: 8 KiB leave 20 waves on a CU, 11 KiB 14, 20 KiB 8; 32 without.  Measured on
+    // MI355X (fraction of 8 TB/s at 32 / 20 / 16 / 14 waves per CU): ring order, 8 bf16 shards
+    // 0.79 / 0.835 / 0.80 / 0.745, 16 bf16 shards 0.77 / 0.81 / 0.81 / 0.765, 64 bf16 shards
+    // 0.76 / 0.79 / 0.79 / 0.77, 32 fp32 shards 0.76 / 0.81 / 0.82 / 0.84; halving order, 8 bf16 and
+    // 16 fp32 shards 0.76 / 0.785 / 0.79 / 0.80, 64 bf16 shards 0.77 at 32 ... 14 and 0.79 at 8.
+    // Launches below 512 MiB of traffic are too short to profit.
+    if (traffic < ((size_t)512 << 20)) return 0;
+    if (order == PCCL_HIP_ORDER_RING) return f32 && k >= 24 ? 11264 : 8192;
+    return k >= 32 ? 20480 : 11264;
+  }
   if (order == PCCL_HIP_ORDER_RING) {
     if (g >= k) {
       if (f32) return k >= 24 ? (traffic >= ((size_t)768 << 20) ? 49152 : 32768) : k >= 16 ? 32768 : k >= 5 ? 24576 : 0;
@@ -529,12 +551,17 @@ long kway_lds_pad(int k, int g, int dtype, int order, size_t traffic) {
 int launch_kway(const KwayArgs& args, int k, int g, int nout, size_t n, int dtype, int order,
                 int first0, int per_hop, hipStream_t stream, const char* what) {
   if (n == 0 || nout == 0) return PCCL_HIP_OK;
+  const size_t traffic = ((size_t)k + 1) * n * esize_of(dtype) * (size_t)nout;
+  const Tune tune = current_tune(false, traffic);
+  long wg = g_wg_kway.load(std::memory_order_relaxed);
+  if (wg < 0) wg = stream_hint(-1, traffic) ? kRowThreads : kThreads;
+  if (!(tune.ntl && tune.nts)) wg = kThreads;   // the one-wave variant exists for non-temporal streams only
   long pad = g_lds_pad_kway.load(std::memory_order_relaxed);
-  if (pad < 0) pad = kway_lds_pad(k, g, dtype, order, ((size_t)k + 1) * n * esize_of(dtype) * (size_t)nout);
-  KwayLaunch l{&args, k, g, nout, dtype, order, first0, per_hop, n, tiles_for(n * esize_of(dtype), 1),
-               (unsigned)pad, stream};
+  if (pad < 0) pad = kway_lds_pad(k, g, dtype, order, traffic, (int)wg);
+  KwayLaunch l{&args, k, g, nout, dtype, order, first0, per_hop, n, tiles_for(n * esize_of(dtype), 1, (int)wg),
+               (unsigned)pad, (int)wg, stream};
   if (int rc = check_work_items((size_t)nout, l.tiles, what)) return rc;
-  with_tuning(current_tune(false, ((size_t)k + 1) * n * esize_of(dtype) * (size_t)nout), l);
+  with_tuning(tune, l);
   return launch_status(what);
 }
 
@@ -624,6 +651,10 @@ int pccl_hip_set_tuning(const char* key, long value) {
     if (value != 1 && value != 2 && value != 4 && value != 8)
       return fail(PCCL_HIP_EINVAL, "set_tuning: unroll must be 1, 2, 4 or 8");
     g_unroll = value;
+  } else if (!strcmp(key, "wg_kway")) {
+    if (value != -1 && value != 64 && value != 256)
+      return fail(PCCL_HIP_EINVAL, "set_tuning: wg_kway must be -1, 64 or 256");
+    g_wg_kway = value;
   } else if (!strcmp(key, "add_rows")) {
     g_add_rows = value != 0;
   } else if (!strcmp(key, "launch_mib_rows")) {
@@ -672,6 +703,7 @@ long pccl_hip_get_tuning(const char* key) {
   if (!key) return -1;
   if (!strcmp(key, "grid_cap")) return g_grid_cap;
   if (!strcmp(key, "unroll")) return g_unroll;
+  if (!strcmp(key, "wg_kway")) return g_wg_kway;
   if (!strcmp(key, "add_rows")) return g_add_rows;
   if (!strcmp(key, "launch_mib_rows")) return g_launch_mib_rows;
   if (!strcmp(key, "unroll_copy")) return g_unroll_copy;

@@ -886,12 +886,12 @@ constexpr int tree_group() { return K >= 32 ? 8 : 4; }
 constexpr int kFoldBatch = 2;
 constexpr int kFoldPairedFrom = 16;
 
-template <class Acc, int L, class Load>
+template <class Acc, int L, int PF = kFoldPairedFrom, class Load>
 __device__ __forceinline__ void ring_fold(Load&& load, int count, int first, float* acc) {
   int q = first;
   load(q, acc);
   int done = 1;
-  if (count >= kFoldPairedFrom) {
+  if (count >= PF) {
     for (; done + kFoldBatch <= count; done += kFoldBatch) {
       float f[kFoldBatch][L];
 #pragma unroll
@@ -922,12 +922,12 @@ __device__ __forceinline__ void ring_fold(Load&& load, int count, int first, flo
 //   K >= 2 : halving order for k == K: leaves v[m] = shard[first ^ m] summed by
 //            the butterfly v[m] += v[m+h], h = K/2 .. 1, evaluated depth first
 //            by tree_sum (the same tree with only log2 K live partial sums).
-template <class Acc, int K, int L, class Load>
+template <class Acc, int K, int L, int PF = kFoldPairedFrom, class Load>
 __device__ __forceinline__ void fold_shards(Load&& load, int k, int g, int first, int first_outer,
                                             float* acc) {
   if constexpr (K == 0) {
     if (g >= k) {
-      ring_fold<Acc, L>(load, k, first, acc);
+      ring_fold<Acc, L, PF>(load, k, first, acc);
     } else {
       // two-level ring: shards form k/g groups of g; every group is folded in
       // ring order from `first`, and the group sums are folded in ring order
@@ -937,7 +937,7 @@ __device__ __forceinline__ void fold_shards(Load&& load, int k, int g, int first
       int go = first_outer;
       for (int og = 0; og < groups; ++og) {
         float part[L];
-        ring_fold<Acc, L>([&](int q, float* f) { load(go * g + q, f); }, g, first, part);
+        ring_fold<Acc, L, PF>([&](int q, float* f) { load(go * g + q, f); }, g, first, part);
         if (og == 0) {
 #pragma unroll
           for (int l = 0; l < L; ++l) acc[l] = part[l];
@@ -957,8 +957,8 @@ __device__ __forceinline__ void fold_shards(Load&& load, int k, int g, int first
 // (first0 + j) mod k (or, for the two-level ring, at the inner and outer
 // successors of j).  Output and shards may start at any element alignment;
 // the few elements around the vector body go one by one through the same fold.
-template <class Acc, int K, int U, bool NTL, bool NTS>
-__global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int g, int nout,
+template <class Acc, int K, int U, bool NTL, bool NTS, int T = kThreads, int PF = kFoldPairedFrom>
+__global__ __launch_bounds__(T) void k_reduce_kway(KwayArgs t, int k, int g, int nout,
                                                           size_t n, int first0,
                                                           size_t tiles_per_seg, Span span) {
   typedef typename Acc::op Op;
@@ -984,14 +984,14 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
     size_t head = (mis % sizeof(elem)) == 0 ? ((16u - mis) & 15u) / sizeof(elem) : n;
     if (head > n) head = n;
     const size_t nvec = (n - head) / Op::kPerVec;
-    const size_t base = tile * (size_t)(kThreads * U);
+    const size_t base = tile * (size_t)(T * U);
 
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const size_t v = base + (size_t)u * kThreads + tid;
+      const size_t v = base + (size_t)u * T + tid;
       // an address is a workgroup-uniform 64-bit base plus a 32-bit lane offset:
       // the unrolled folds then need no vector registers for their k addresses
-      const size_t wg_byte = (eoff + head) * sizeof(elem) + (base + (size_t)u * kThreads) * 16;
+      const size_t wg_byte = (eoff + head) * sizeof(elem) + (base + (size_t)u * T) * 16;
       const uint32_t lane_byte = tid * 16u;
       if constexpr (K >= 16 && Acc::kPacked) {
         if (v < nvec) {
@@ -1020,7 +1020,7 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
       } else
       if (v < nvec) {
         float acc[L];
-        fold_shards<Acc, K, L>(
+        fold_shards<Acc, K, L, PF>(
             [&](int q, float* f) {
               Acc::widen(ld16u<NTL>((const uint8_t*)t.shard[q] + wg_byte + lane_byte), f);
             },
@@ -1032,7 +1032,7 @@ __global__ __launch_bounds__(kThreads) void k_reduce_kway(KwayArgs t, int k, int
     // head and tail, by the first tile of the output
     const size_t body_end = head + nvec * Op::kPerVec;
     const size_t loose = tile == 0 ? head + (n - body_end) : 0;
-    for (size_t e = tid; e < loose; e += kThreads) {
+    for (size_t e = tid; e < loose; e += T) {
       const size_t i = e < head ? e : body_end + (e - head);
       float acc1[1];
       fold_shards<Acc, K, 1>(

@@ -460,3 +460,106 @@ def test_reduce_kway_special_values(target, dtype, k, order):
         assert np.array_equal(np.isnan(got), np.isnan(want))
         got, want = np.where(np.isnan(got), np.float32(0), got), np.where(np.isnan(want), np.float32(0), want)
     assert_bits_equal(got, want, "reduce_kway special values")
+
+
+def _fold_want(shards, dtype, order, first):
+    k = len(shards)
+    if order == "ring":
+        want = shards[first]
+        for t in range(1, k):
+            want = O.vector_add(want, shards[(first + t) % k], dtype)
+        return want
+    v = [shards[first ^ m] for m in range(k)]
+    h = k // 2
+    while h >= 1:
+        for m in range(h):
+            v[m] = O.vector_add(v[m], v[m + h], dtype)
+        h //= 2
+    return v[0]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("order", ["ring", "halving"])
+def test_one_wave_fold_gives_the_same_bits(target, dtype, order):
+    """The fused reduce with one-wave workgroups and paired loads (what streams
+    from HBM get; forced here at test sizes): every k, shards at any alignment,
+    whole reduce_scatters flat and on a grid."""
+    import torch
+    from pccl import kernels
+    lib = target.native
+    saved = {k: lib.get_tuning(k) for k in ("wg_kway", "nt_load", "nt_store", "lds_pad_kway")}
+    try:
+        lib.set_tuning("wg_kway", 64)
+        lib.set_tuning("nt_load", 1)
+        lib.set_tuning("nt_store", 1)
+        for pad in (0, 8192):
+            lib.set_tuning("lds_pad_kway", pad)
+            for k in (2, 3, 4, 7, 8, 16, 17, 32, 64):
+                if order == "halving" and k & (k - 1):
+                    continue
+                n = 3001 if k < 32 else 1037
+                shards = make_inputs(k, n, dtype, seed=100 + k)
+                shifts = [(3 * q + 1) % 8 if pad else 0 for q in range(k)]      # second pass: every shard at its own alignment
+                bufs = [to_torch(np.concatenate([np.zeros(sh, x.dtype), x, np.zeros(8 - sh, x.dtype)]), dtype, target.device)
+                        for x, sh in zip(shards, shifts)]
+                ts = [b[sh:sh + n] for b, sh in zip(bufs, shifts)]
+                out_big = torch.zeros(n + 8, dtype=ts[0].dtype, device=target.device)
+                out = out_big[(3 if pad else 0):][:n]
+                first = (k // 3) % k
+                print(f"one-wave fold dtype={dtype} order={order} k={k} pad={pad}", flush=True)
+                lib.reduce_kway(out.data_ptr(), [t.data_ptr() for t in ts], n, CODE[dtype], 0 if order == "ring" else 1,
+                                first, True, target.stream())
+                target.sync()
+                assert_bits_equal(to_numpy(out.clone(), dtype), _fold_want(shards, dtype, order, first), f"k={k} pad={pad}")
+        alg = "ring" if order == "ring" else "recursive"
+        for P, B in ((4, 9001), (8, 515)):
+            ins = make_inputs(P, P * B, dtype, seed=31 + P)
+            t_in = [to_torch(x, dtype, target.device) for x in ins]
+            want = (O.ring_reduce_scatter if order == "ring" else O.recursive_halving_reduce_scatter)(ins, dtype)
+            t_out = [torch.zeros(B, dtype=t_in[0].dtype, device=target.device) for _ in range(P)]
+            kernels.reduce_scatter_ranks(t_out, t_in, alg, "fused")
+            target.sync()
+            for r in range(P):
+                assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"{alg} P={P} rank {r}")
+            want2 = O.reduce_scatter_2d(ins, 2, P // 2, dtype, alg)
+            kernels.reduce_scatter_2d_ranks(t_out, t_in, 2, P // 2, alg, "fused")
+            target.sync()
+            for r in range(P):
+                assert_bits_equal(to_numpy(t_out[r], dtype), want2[r], f"2-D {alg} 2x{P // 2} rank {r}")
+    finally:
+        for k, v in saved.items():
+            lib.set_tuning(k, v)
+
+
+@pytest.mark.parametrize("add_rows,launch_mib_rows", [(0, 0), (1, 1), (1, 3)])
+def test_lean_and_general_add_kernels_agree(target, add_rows, launch_mib_rows):
+    """Aligned contiguous adds go to the lean one-wave kernels, everything else
+    (and everything when add_rows = 0) to the general ones; a lean step cut into
+    several launches between rows (3 MiB) or inside rows (1 MiB) computes the same."""
+    import torch
+    from pccl import kernels
+    lib = target.native
+    saved = {k: lib.get_tuning(k) for k in ("add_rows", "launch_mib_rows")}
+    try:
+        lib.set_tuning("add_rows", add_rows)
+        lib.set_tuning("launch_mib_rows", launch_mib_rows)
+        P, B = 4, 150_000          # blocks of whole vectors: the aligned path
+        for dtype in DTYPES:
+            ins = make_inputs(P, P * B, dtype, seed=29)
+            t_in = [to_torch(x, dtype, target.device) for x in ins]
+            for alg, ref in (("ring", O.ring_reduce_scatter), ("recursive", O.recursive_halving_reduce_scatter)):
+                want = ref(ins, dtype)
+                for mode in ("steps", "faithful"):
+                    t_out = [torch.zeros(B, dtype=t_in[0].dtype, device=target.device) for _ in range(P)]
+                    kernels.reduce_scatter_ranks(t_out, t_in, alg, mode)
+                    target.sync()
+                    for r in range(P):
+                        assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"{alg}/{mode}/{dtype} rank {r}")
+            a, b = ins[0], ins[1]
+            ta, tb = to_torch(a, dtype, target.device), to_torch(b, dtype, target.device)
+            kernels.accumulate(ta, tb)
+            target.sync()
+            assert_bits_equal(to_numpy(ta, dtype), O.vector_add(a, b, dtype), "accumulate")
+    finally:
+        for k, v in saved.items():
+            lib.set_tuning(k, v)
