@@ -33,6 +33,8 @@ Workloads:
         from the loads to the stores (2:1, 8:1, 32:1, 1:16)
   sweep  GB/s against message size, 64 MiB .. 2 GiB per operand
   latency  small messages, 4 KiB .. 1 MiB in bf16: microseconds per call
+  placement  the cfg2 shape on six separately allocated groups of buffers in one
+        process: the spread that comes from where the buffers lie physically
   all   (default) cfg2/steps as the headline plus every row above
 
 The CPU baseline (the reference's per-rank algorithm on host cores, one process
@@ -71,7 +73,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="all", choices=["all"] + WORKLOADS + ["latency", "ceilings", "sweep"])
+    ap.add_argument("--workload", default="all", choices=["all"] + WORKLOADS + ["latency", "ceilings", "sweep", "placement"])
     ap.add_argument("--mode", default=None, choices=["steps", "fused", "faithful"],
                     help="execution mode of the collective (default: per-step replay for the reductions, "
                          "one fused launch for cfg4, cfg4u and cfg5)")
@@ -672,6 +674,29 @@ def size_sweep(steps, warmup, device):
     return rows
 
 
+def placement_spread(sets, steps, warmup, device):
+    """The cfg2 shape on `sets` separately allocated groups of rank buffers, all of
+    them alive at once: every group lies on other physical pages, and the same code
+    on the same virtual layout runs at a rate that depends on the group.  Returns,
+    per group, the GB/s of the per-step mode and of the fused mode."""
+    import torch
+    from pccl import _native
+    lib = _native.load()
+    groups, rows = [], []
+    for g in range(sets):
+        groups.append(make_ring_rs(8, 256 * MiB, "bf16", ["steps", "fused"], device, seed=1234 + 100 * g, std=1e-2))
+    for g, built in enumerate(groups):
+        row = {"group": g}
+        for mode in ("steps", "fused"):
+            step, info = built[mode]
+            dev_ms, _, launched = time_steps(step, steps, warmup, lib)
+            ms = dev_ms / steps
+            row[mode + "_GBps"] = round(info["alg_bytes"] / (ms * 1e-3) / 1e9, 1)
+            row[mode + "_frac"] = round(row[mode + "_GBps"] / HBM_PEAK_GBPS, 4)
+        rows.append(row)
+    return rows
+
+
 def latency_sweep(steps, warmup, device):
     """Microseconds per call for launch-bound message sizes (bf16), through the
     ordinary Python API unless a column says otherwise."""
@@ -904,6 +929,21 @@ def main():
             "config": {"workload": "sweep: GB/s against message size (MiB per operand); value = mean accumulate "
                                    "bf16 at >= 256 MiB", "GBps": rows,
                        "pct_of_hbm_peak": round(100 * val / HBM_PEAK_GBPS, 2)},
+            "roofline": None, "cpu_baseline": None}), flush=True)
+        return 0
+
+    if args.workload == "placement":
+        rows = placement_spread(6, min(args.steps, 10), min(args.warmup, 3), device)
+        vals = [r["steps_GBps"] for r in rows]
+        val = round(sum(vals) / len(vals), 1)
+        print(json.dumps({
+            "metric": METRIC, "value": val, "unit": "GB/s", "n_gpus": 1, "steps": min(args.steps, 10),
+            "warmup": min(args.warmup, 3), "ms_per_step": None, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "placement: cfg2 (ring reduce_scatter, P=8, bf16, 512 MiB per rank) on six separately "
+                                   "allocated groups of buffers; value = mean of the per-step mode", "groups": rows,
+                       "steps_min_max": [min(vals), max(vals)],
+                       "fused_min_max": [min(r["fused_GBps"] for r in rows), max(r["fused_GBps"] for r in rows)]},
             "roofline": None, "cpu_baseline": None}), flush=True)
         return 0
 

@@ -15,6 +15,7 @@
 // No MFMA: there is no contraction anywhere on this path.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cstdarg>
 #include <cstdint>
@@ -39,12 +40,35 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+// The status of a launch is what the launch call itself returns: hipGetLastError()
+// would hand out (and clear) whatever an earlier, unrelated call of this thread
+// left behind, and a caller's own check could eat ours.  The first failure of a
+// call's launches is kept per thread until launch_status() reports it.
+thread_local hipError_t t_launch_error = hipSuccess;
+
+inline void note_launch(hipError_t e) {
+  if (e != hipSuccess && t_launch_error == hipSuccess) t_launch_error = e;
+}
+
 int launch_status(const char* what) {
-  hipError_t e = hipGetLastError();
+  const hipError_t e = t_launch_error;
+  t_launch_error = hipSuccess;
   if (e != hipSuccess)
     return fail(PCCL_HIP_ELAUNCH, "%s: launch failed: %s", what, hipGetErrorString(e));
   return PCCL_HIP_OK;
 }
+
+#ifndef PCCL_LAUNCH   // a host stand-in for the HIP runtime brings its own
+template <class T> struct same_as { typedef T type; };
+template <class... P>
+hipError_t launch_kernel(void (*kernel)(P...), dim3 grid, dim3 block, unsigned lds, hipStream_t stream,
+                         typename same_as<P>::type... args) {
+  void* ptrs[] = {(void*)&args...};
+  return hipLaunchKernel((const void*)kernel, grid, block, ptrs, lds, stream);
+}
+#define PCCL_LAUNCH(kernel, grid, block, lds, stream, ...) \
+  note_launch(launch_kernel(kernel, grid, block, lds, stream, __VA_ARGS__))
+#endif
 
 std::atomic<long> g_grid_cap{0};
 std::atomic<long> g_unroll{4};        // vectors per thread and operand, general add kernels
@@ -230,9 +254,9 @@ struct AddLaunch {
     const unsigned lds = (unsigned)g_lds_pad.load();
     for_spans((size_t)count * pc.s1 * pc.s2 * tiles, (size_t)3 * T * 16 * U, 1, add_launch_mib(), [&](Span span, unsigned grid) {
       if (dtype == PCCL_HIP_F32)
-        hipLaunchKernelGGL((k_add_segs<OpF32, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *segs, count, pc, tiles, aligned, span);
+        PCCL_LAUNCH((k_add_segs<OpF32, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *segs, count, pc, tiles, aligned, span);
       else
-        hipLaunchKernelGGL((k_add_segs<OpBF16, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *segs, count, pc, tiles, aligned, span);
+        PCCL_LAUNCH((k_add_segs<OpBF16, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *segs, count, pc, tiles, aligned, span);
     });
   }
   template <int U, bool NTL, bool NTS>
@@ -280,7 +304,7 @@ void launch_add_rows(const AddSegs& segs, int count, size_t n, int dtype, const 
   const size_t tiles = (nvec + kRowThreads - 1) / kRowThreads;
   for_rows(count, tiles, (size_t)3 * kRowThreads * 16, g_launch_mib_rows.load(std::memory_order_relaxed),
            [&](int row0, int nrows, uint32_t tile0, unsigned ntiles) {
-#define PCCL_ROWS(OP, L, S) hipLaunchKernelGGL((k_add_rows<OP, L, S>), dim3(ntiles, (unsigned)nrows), dim3(kRowThreads), 0, stream, segs, row0, nvec, tile0)
+#define PCCL_ROWS(OP, L, S) PCCL_LAUNCH((k_add_rows<OP, L, S>), dim3(ntiles, (unsigned)nrows), dim3(kRowThreads), 0, stream, segs, row0, nvec, tile0)
     if (dtype == PCCL_HIP_F32) {
       if (t.ntl) { if (t.nts) PCCL_ROWS(OpF32, true, true); else PCCL_ROWS(OpF32, true, false); }
       else { if (t.nts) PCCL_ROWS(OpF32, false, true); else PCCL_ROWS(OpF32, false, false); }
@@ -344,7 +368,7 @@ struct CopyLaunch {
   void operator()() const {
     const unsigned lds = copy_lds_pad(traffic);
     for_spans((size_t)count * tiles, 2 * kTileBytes * U, 1, 0, [&](Span span, unsigned grid) {
-      hipLaunchKernelGGL((k_copy_segs<U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *segs, count, tiles, aligned, span);
+      PCCL_LAUNCH((k_copy_segs<U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *segs, count, tiles, aligned, span);
     });
   }
 };
@@ -377,7 +401,7 @@ struct CopyPiecesLaunch {
   void operator()() const {
     const unsigned lds = copy_lds_pad(2 * (size_t)count * pc.s1 * pc.s2 * pc.len);
     for_spans((size_t)count * pc.s1 * pc.s2 * tiles, 2 * kTileBytes * U, 1, 0, [&](Span span, unsigned grid) {
-      hipLaunchKernelGGL((k_copy_pieces<U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *segs, count, pc, tiles, aligned, span);
+      PCCL_LAUNCH((k_copy_pieces<U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *segs, count, pc, tiles, aligned, span);
     });
   }
 };
@@ -407,9 +431,9 @@ struct RhLaunch {
     const unsigned lds = (unsigned)g_lds_pad.load();
     for_spans((size_t)P * tiles, (size_t)3 * T * 16 * U, 1, add_launch_mib(), [&](Span span, unsigned grid) {
       if (dtype == PCCL_HIP_F32)
-        hipLaunchKernelGGL((k_rh_round<OpF32, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *args, P, B, round, from_src, to_outs, tiles, aligned, span);
+        PCCL_LAUNCH((k_rh_round<OpF32, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *args, P, B, round, from_src, to_outs, tiles, aligned, span);
       else
-        hipLaunchKernelGGL((k_rh_round<OpBF16, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *args, P, B, round, from_src, to_outs, tiles, aligned, span);
+        PCCL_LAUNCH((k_rh_round<OpBF16, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *args, P, B, round, from_src, to_outs, tiles, aligned, span);
     });
   }
   template <int U, bool NTL, bool NTS>
@@ -432,9 +456,9 @@ struct GatherLaunch {
     const size_t item_bytes = kTileBytes * U * (1 + ((size_t)nout + split - 1) / split);
     for_spans((size_t)P * tiles * (size_t)split, item_bytes, (size_t)split, 0, [&](Span span, unsigned grid) {
       if (nt)
-        hipLaunchKernelGGL((k_gather_multicast<U, false, true>), dim3(grid), dim3(kThreads), lds_pad, stream, *args, P, nout, tiles, split, span);
+        PCCL_LAUNCH((k_gather_multicast<U, false, true>), dim3(grid), dim3(kThreads), lds_pad, stream, *args, P, nout, tiles, split, span);
       else
-        hipLaunchKernelGGL((k_gather_multicast<U, false, false>), dim3(grid), dim3(kThreads), lds_pad, stream, *args, P, nout, tiles, split, span);
+        PCCL_LAUNCH((k_gather_multicast<U, false, false>), dim3(grid), dim3(kThreads), lds_pad, stream, *args, P, nout, tiles, split, span);
     });
   }
 };
@@ -448,7 +472,7 @@ struct TransposeLaunch {
   template <int U, bool NTL, bool NTS>
   void operator()() const {
     for_spans(rows * cols * tiles, 2 * kTileBytes * U, 1, 0, [&](Span span, unsigned grid) {
-      hipLaunchKernelGGL((k_block_transpose<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, dst, src, rows, cols, m, tiles, aligned, span);
+      PCCL_LAUNCH((k_block_transpose<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, dst, src, rows, cols, m, tiles, aligned, span);
     });
   }
 };
@@ -468,7 +492,7 @@ struct KwayLaunch {
   void run_wg(long span_mib) const {
     static_assert(U == 1, "the fused reduce is launched with one vector per thread");
 #define PCCL_KWAY(KV) \
-  hipLaunchKernelGGL((k_reduce_kway<Acc, KV, U, NTL, NTS, T, PF>), dim3(grid), dim3(T), lds_pad, stream, *args, k, g, nout, n, first0, tiles, span)
+  PCCL_LAUNCH((k_reduce_kway<Acc, KV, U, NTL, NTS, T, PF>), dim3(grid), dim3(T), lds_pad, stream, *args, k, g, nout, n, first0, tiles, span)
     for_spans((size_t)nout * tiles, (size_t)T * 16 * U * ((size_t)k + 1), 1, span_mib, [&](Span span, unsigned grid) {
       if (order == PCCL_HIP_ORDER_RING) { PCCL_KWAY(0); return; }
       switch (k) {
@@ -526,15 +550,15 @@ long kway_lds_pad(int k, int g, int dtype, int order, size_t traffic, int thread
   if (!stream_hint(-1, traffic)) return 0;
   const bool f32 = dtype == PCCL_HIP_F32;
   if (threads == kRowThreads) {
-    // One-wave workgroups: 8 KiB leave 20 waves on a CU, 11 KiB 14, 20 KiB 8; 32 without.  Measured on
+    // One-wave workgroups: 8 KiB leave 20 waves on a CU, 11 KiB 14, 16 KiB 10; 32 without.  Measured on
     // MI355X (fraction of 8 TB/s at 32 / 20 / 16 / 14 waves per CU): ring order, 8 bf16 shards
     // 0.79 / 0.835 / 0.80 / 0.745, 16 bf16 shards 0.77 / 0.81 / 0.81 / 0.765, 64 bf16 shards
     // 0.76 / 0.79 / 0.79 / 0.77, 32 fp32 shards 0.76 / 0.81 / 0.82 / 0.84; halving order, 8 bf16 and
-    // 16 fp32 shards 0.76 / 0.785 / 0.79 / 0.80, 64 bf16 shards 0.77 at 32 ... 14 and 0.79 at 8.
-    // Launches below 512 MiB of traffic are too short to profit.
+    // 16 fp32 shards 0.76 / 0.785 / 0.79 / 0.80, 64 bf16 shards of 1 GiB 0.79 / 0.81 / - / 0.855 (and
+    // 0.855 at 10, 0.80 at 8).  Launches below 512 MiB of traffic are too short to profit.
     if (traffic < ((size_t)512 << 20)) return 0;
     if (order == PCCL_HIP_ORDER_RING) return f32 && k >= 24 ? 11264 : 8192;
-    return k >= 32 ? 20480 : 11264;
+    return 11264;
   }
   if (order == PCCL_HIP_ORDER_RING) {
     if (g >= k) {
@@ -612,6 +636,88 @@ int launch_copy_list(const RankList<CopyItem>& list, hipStream_t stream, const c
     if (int rc = launch_copy(segs, cnt, stream, what)) return rc;
   }
   return PCCL_HIP_OK;
+}
+
+// ---------------------------------------------------------------------------
+// overlap of the buffers of one call
+// ---------------------------------------------------------------------------
+// A collective reads some buffers (inputs) and writes others (outputs, work
+// space).  Readers may share memory among themselves; a written buffer may
+// share memory with nothing, with ONE exception per rank that the kernels
+// handle element by element (every element is read by the thread that
+// overwrites it, and by no other): the in-place use the reference allows
+// because it copies first (pccl/src/reduce_scatter.cpp:119-123,
+// pccl/src/all_gather.cpp:31-35) -- a reduce_scatter output that IS block r of
+// rank r's input, an all_gather shard that IS block r of rank r's output.
+struct Extent {
+  uintptr_t lo, hi;   // [lo, hi)
+  int rank;           // index within its table
+  char kind;          // 'i' read only, 'o' output, 'w' work space
+  bool in_place;      // this written buffer coincides with its rank's reader exactly where the kernels allow it
+};
+
+class ExtentList {
+ public:
+  void add(const void* p, size_t bytes, int rank, char kind, bool in_place = false) {
+    if (!p || bytes == 0) return;
+    Extent e{(uintptr_t)p, (uintptr_t)p + bytes, rank, kind, in_place};
+    if (n_ < kSmall) small_[n_++] = e;
+    else { if (big_.empty()) big_.assign(small_, small_ + n_); big_.push_back(e); ++n_; }
+  }
+  // 0 if the call's buffers overlap only where that is allowed, else EINVAL with a message naming two of them
+  int check(const char* what) {
+    Extent* v = big_.empty() ? small_ : big_.data();
+    std::sort(v, v + n_, [](const Extent& a, const Extent& b) { return a.lo != b.lo ? a.lo < b.lo : a.kind < b.kind; });
+    // sweep by start address; `top` is the started extent that reaches farthest
+    // among the writers and among the readers, `partner` the one reader a writer
+    // may coincide with (or the one writer a reader may lie in)
+    const Extent* topw = nullptr;
+    const Extent* topr = nullptr;
+    for (size_t i = 0; i < n_; ++i) {
+      const Extent& x = v[i];
+      const bool xw = x.kind != 'i';
+      if (topw && topw->hi > x.lo) {           // a writer is still open here
+        const Extent& w = *topw;
+        const bool ok = !xw && w.in_place && w.kind == 'o' && x.rank == w.rank && pairs(x, w);
+        if (!ok) return clash(what, w, x);
+      }
+      if (xw && topr && topr->hi > x.lo) {     // a reader is still open where this writer starts
+        const Extent& r = *topr;
+        const bool ok = x.in_place && x.kind == 'o' && r.rank == x.rank && pairs(r, x);
+        if (!ok) return clash(what, r, x);
+        // no second reader may reach into it either: the readers that started before the top one
+        for (size_t j = 0; j < i; ++j)
+          if (v[j].kind == 'i' && &v[j] != topr && v[j].hi > x.lo) return clash(what, v[j], x);
+      }
+      if (xw) { if (!topw || x.hi > topw->hi) topw = &x; }
+      else { if (!topr || x.hi > topr->hi) topr = &x; }
+    }
+    return PCCL_HIP_OK;
+  }
+
+ private:
+  // one of the two contains the other: the only shape an allowed pair has
+  static bool pairs(const Extent& r, const Extent& w) {
+    return (r.lo <= w.lo && w.hi <= r.hi) || (w.lo <= r.lo && r.hi <= w.hi);
+  }
+  static const char* name(char kind) { return kind == 'i' ? "inputs" : kind == 'o' ? "outputs" : "work"; }
+  static int clash(const char* what, const Extent& a, const Extent& b) {
+    return fail(PCCL_HIP_EINVAL,
+                "%s: %s[%d] and %s[%d] overlap in memory (a written buffer may share memory with nothing, except "
+                "outputs[r] being exactly block r of inputs[r] in a reduce_scatter, or inputs[r] being exactly block r "
+                "of outputs[r] in an all_gather)",
+                what, name(a.kind), a.rank, name(b.kind), b.rank);
+  }
+  static constexpr size_t kSmall = 3 * (size_t)PCCL_HIP_MAX_RANKS;
+  Extent small_[kSmall];
+  std::vector<Extent> big_;
+  size_t n_ = 0;
+};
+
+// two buffers of `bytes` bytes that share memory without being the same buffer
+bool partly_overlap(const void* p, const void* q, size_t bytes) {
+  const uintptr_t a = (uintptr_t)p, b = (uintptr_t)q;
+  return a != b && a < b + bytes && b < a + bytes;
 }
 
 bool pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
@@ -727,6 +833,8 @@ int pccl_hip_add(void* dst, const void* a, const void* b, size_t n, int dtype, v
   if (int rc = check_dtype(dtype, what)) return rc;
   if (n == 0) return PCCL_HIP_OK;
   if (!dst || !a || !b) return fail(PCCL_HIP_EINVAL, "%s: NULL operand", what);
+  if (partly_overlap(dst, a, n * esize_of(dtype)) || partly_overlap(dst, b, n * esize_of(dtype)))
+    return fail(PCCL_HIP_EINVAL, "%s: dst may be a or b exactly, but overlaps one of them partly", what);
   AddSegs segs;
   segs.dst[0] = dst; segs.a[0] = a; segs.b[0] = b;
   return launch_add(segs, 1, n, dtype, (hipStream_t)stream, what);
@@ -737,6 +845,8 @@ int pccl_hip_accumulate(void* dst, const void* src, size_t n, int dtype, void* s
   if (int rc = check_dtype(dtype, what)) return rc;
   if (n == 0) return PCCL_HIP_OK;
   if (!dst || !src) return fail(PCCL_HIP_EINVAL, "%s: NULL operand", what);
+  if (partly_overlap(dst, src, n * esize_of(dtype)))
+    return fail(PCCL_HIP_EINVAL, "%s: src may be dst exactly, but overlaps it partly", what);
   AddSegs segs;
   segs.dst[0] = dst; segs.a[0] = dst; segs.b[0] = src;
   return launch_add(segs, 1, n, dtype, (hipStream_t)stream, what);
@@ -796,7 +906,7 @@ int pccl_hip_rh_round(void* const* bufs, const void* const* src, void* const* ou
     hipStream_t st = (hipStream_t)stream;
     for_rows(P, tiles, (size_t)3 * kRowThreads * 16, g_launch_mib_rows.load(std::memory_order_relaxed),
              [&](int row0, int nrows, uint32_t tile0, unsigned ntiles) {
-#define PCCL_RH(OP, L, S) hipLaunchKernelGGL((k_rh_rows<OP, L, S>), dim3(ntiles, (unsigned)nrows), dim3(kRowThreads), 0, st, args, row0, log2_group, B, from_src, outs_i, nvec, tile0)
+#define PCCL_RH(OP, L, S) PCCL_LAUNCH((k_rh_rows<OP, L, S>), dim3(ntiles, (unsigned)nrows), dim3(kRowThreads), 0, st, args, row0, log2_group, B, from_src, outs_i, nvec, tile0)
       if (dtype == PCCL_HIP_F32) {
         if (t.ntl) { if (t.nts) PCCL_RH(OpF32, true, true); else PCCL_RH(OpF32, true, false); }
         else { if (t.nts) PCCL_RH(OpF32, false, true); else PCCL_RH(OpF32, false, false); }
@@ -828,6 +938,12 @@ int pccl_hip_reduce_kway(void* out, const void* const* shards, int k, size_t n, 
   if (n == 0) return PCCL_HIP_OK;
   if (!out) return fail(PCCL_HIP_EINVAL, "%s: out is NULL", what);
   if (int rc = check_table(shards, k, what, "shards")) return rc;
+  {
+    ExtentList ext;
+    for (int q = 0; q < k; ++q) ext.add(shards[q], n * esize_of(dtype), q, 'i');
+    ext.add(out, n * esize_of(dtype), 0, 'o');
+    if (int rc = ext.check(what)) return rc;
+  }
   KwayArgs args;
   for (int q = 0; q < k; ++q) args.shard[q] = shards[q];
   args.out[0] = out;
@@ -946,8 +1062,8 @@ int gather_place_all(void* const* outputs, int nout, const void* const* inputs, 
     hipStream_t st = (hipStream_t)stream;
 #define PCCL_STRIPS(UV)                                                                                              \
   case UV:                                                                                                          \
-    if (nts) hipLaunchKernelGGL((k_gather_strips<UV, false, true>), dim3(grid), dim3(kThreads), lds, st, args, P, nout, (uint32_t)n_local, (uint32_t)strip, span); \
-    else hipLaunchKernelGGL((k_gather_strips<UV, false, false>), dim3(grid), dim3(kThreads), lds, st, args, P, nout, (uint32_t)n_local, (uint32_t)strip, span);    \
+    if (nts) PCCL_LAUNCH((k_gather_strips<UV, false, true>), dim3(grid), dim3(kThreads), lds, st, args, P, nout, (uint32_t)n_local, (uint32_t)strip, span); \
+    else PCCL_LAUNCH((k_gather_strips<UV, false, false>), dim3(grid), dim3(kThreads), lds, st, args, P, nout, (uint32_t)n_local, (uint32_t)strip, span);    \
     break;
     for_spans((size_t)P * (size_t)nout * kXcds * n_local, 0, 1, 0, [&](Span span, unsigned grid) {
       switch (U) {
@@ -990,8 +1106,18 @@ int pccl_hip_all_gather_uneven_virtual(void* const* outputs, const void* const* 
   if (!nbytes || !dst_off) return fail(PCCL_HIP_EINVAL, "%s: NULL size table", what);
   if (int rc = check_table((const void* const*)outputs, P, what, "outputs")) return rc;
   if (!inputs) return fail(PCCL_HIP_EINVAL, "%s: inputs is NULL", what);
-  size_t total = 0;
-  for (int k = 0; k < P; ++k) total += nbytes[k];
+  size_t total = 0, end = 0;
+  for (int k = 0; k < P; ++k) {
+    total += nbytes[k];
+    if (nbytes[k] && dst_off[k] + nbytes[k] > end) end = dst_off[k] + nbytes[k];
+  }
+  {
+    ExtentList ext;
+    for (int k = 0; k < P; ++k) ext.add(inputs[k], nbytes[k], k, 'i');
+    for (int k = 0; k < P; ++k)
+      ext.add(outputs[k], end, k, 'o', nbytes[k] != 0 && inputs[k] == (const uint8_t*)outputs[k] + dst_off[k]);
+    if (int rc = ext.check(what)) return rc;
+  }
   CallBytes footprint(((size_t)P + 1) * total);   // P shards and P outputs holding all of them
   // one launch places up to kMaxSeg shards into up to kMaxSeg outputs
   for (int k0 = 0; k0 < P; k0 += kMaxSeg) {
@@ -1042,6 +1168,18 @@ int reduce_scatter_ranks(void* const* outputs, const void* const* inputs, void* 
   if (B == 0) return PCCL_HIP_OK;
   hipStream_t st = (hipStream_t)stream;
   const size_t es = esize_of(dtype);
+  {
+    // In place (outputs[r] is block r of inputs[r]) every mode reads an element before the same thread
+    // overwrites it, except the fused ring beyond the shards of one launch: its chain of launches keeps the
+    // running sum in outputs[r] while block r of inputs[r] is still to come as the last operand.
+    const bool chained = mode == PCCL_HIP_MODE_FUSED && ring && P > kMaxSeg;
+    ExtentList ext;
+    for (int r = 0; r < P; ++r) ext.add(inputs[r], (size_t)P * B * es, r, 'i');
+    for (int r = 0; r < P; ++r)
+      ext.add(outputs[r], B * es, r, 'o', !chained && outputs[r] == (const uint8_t*)inputs[r] + (size_t)r * B * es);
+    if (need_work) for (int r = 0; r < P; ++r) ext.add(work[r], (size_t)P * B * es, r, 'w');
+    if (int rc = ext.check(what)) return rc;
+  }
   // inputs, the work buffers if the mode uses them, and the outputs
   CallBytes footprint(((need_work ? 2 : 1) * (size_t)P * P + P) * B * es);
 
@@ -1250,6 +1388,13 @@ int pccl_hip_all_gather_virtual(void* const* outputs, const void* const* inputs,
   if (int rc = check_table(inputs, P, what, "inputs")) return rc;
   if (block_bytes == 0) return PCCL_HIP_OK;
   hipStream_t st = (hipStream_t)stream;
+  {
+    ExtentList ext;
+    for (int r = 0; r < P; ++r) ext.add(inputs[r], block_bytes, r, 'i');
+    for (int r = 0; r < P; ++r)
+      ext.add(outputs[r], (size_t)P * block_bytes, r, 'o', inputs[r] == (const uint8_t*)outputs[r] + (size_t)r * block_bytes);
+    if (int rc = ext.check(what)) return rc;
+  }
   CallBytes footprint(((size_t)P * P + P) * block_bytes);   // P shards and P outputs of P blocks
 
   if (mode == PCCL_HIP_MODE_FUSED) {
@@ -1324,6 +1469,16 @@ int pccl_hip_reduce_scatter_2d_virtual(void* const* outputs, const void* const* 
   if (m == 0) return PCCL_HIP_OK;
   hipStream_t st = (hipStream_t)stream;
   const size_t es = esize_of(dtype);
+  {
+    const bool steps = mode == PCCL_HIP_MODE_STEPS;
+    ExtentList ext;
+    for (int w = 0; w < W; ++w) ext.add(inputs[w], (size_t)W * m * es, w, 'i');
+    for (int w = 0; w < W; ++w)
+      ext.add(outputs[w], m * es, w, 'o', outputs[w] == (const uint8_t*)inputs[w] + (size_t)w * m * es);
+    if (steps && (intra > 2 || inter > 2) && work) for (int w = 0; w < W; ++w) ext.add(work[w], (size_t)W * m * es, w, 'w');
+    if (steps && intra > 1 && inter > 1 && mid) for (int w = 0; w < W; ++w) ext.add(mid[w], (size_t)inter * m * es, w, 'w');
+    if (int rc = ext.check(what)) return rc;
+  }
   // inputs of W*m elements per rank, as much work space in the per-step mode, the outputs
   CallBytes footprint(((mode == PCCL_HIP_MODE_FUSED ? 1 : 2) * (size_t)W * W + W) * m * es);
   auto at = [es](const void* p, size_t elems) { return (const void*)((const uint8_t*)p + elems * es); };
@@ -1481,6 +1636,14 @@ int pccl_hip_all_gather_2d_virtual(void* const* outputs, const void* const* inpu
   const size_t n = block_bytes;
   if (n == 0) return PCCL_HIP_OK;
   hipStream_t st = (hipStream_t)stream;
+  {
+    ExtentList ext;
+    for (int w = 0; w < W; ++w) ext.add(inputs[w], n, w, 'i');
+    for (int w = 0; w < W; ++w) ext.add(outputs[w], (size_t)W * n, w, 'o', inputs[w] == (const uint8_t*)outputs[w] + (size_t)w * n);
+    if (mode == PCCL_HIP_MODE_STEPS && intra > 1 && inter > 1 && mid)
+      for (int w = 0; w < W; ++w) ext.add(mid[w], (size_t)inter * n, w, 'w');
+    if (int rc = ext.check(what)) return rc;
+  }
   CallBytes footprint(((size_t)W * W + W) * n);   // W shards and W outputs of W blocks
 
   if (W == 1) {
@@ -1582,10 +1745,10 @@ int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream) {
   if (tiles > kMaxGrid) return fail(PCCL_HIP_EINVAL, "%s: buffer too large", what);
   hipStream_t st = (hipStream_t)stream;
   if (kind == 0)
-    hipLaunchKernelGGL((k_probe_read<4, true>), dim3((unsigned)tiles), dim3(kThreads), 0, st,
+    PCCL_LAUNCH((k_probe_read<4, true>), dim3((unsigned)tiles), dim3(kThreads), 0, st,
                        (const u32x4*)buf, (u32x4*)buf, nvec);
   else
-    hipLaunchKernelGGL((k_probe_write<1, false>), dim3((unsigned)tiles), dim3(kThreads), 0, st, (u32x4*)buf, nvec,
+    PCCL_LAUNCH((k_probe_write<1, false>), dim3((unsigned)tiles), dim3(kThreads), 0, st, (u32x4*)buf, nvec,
                        0x3f803f80u);
   g_launches.fetch_add(1, std::memory_order_relaxed);
   return launch_status(what);
@@ -1612,9 +1775,9 @@ int pccl_hip_probe_mix(const void* const* reads, int nr, void* const* writes, in
   hipStream_t st = (hipStream_t)stream;
   const unsigned grid = (unsigned)tiles;
   switch (vectors) {
-    case 1: hipLaunchKernelGGL((k_probe_mix<1, true, true>), dim3(grid), dim3(kThreads), 0, st, args, nr, nw, nvec, shape, 0x3f803f80u); break;
-    case 2: hipLaunchKernelGGL((k_probe_mix<2, true, true>), dim3(grid), dim3(kThreads), 0, st, args, nr, nw, nvec, shape, 0x3f803f80u); break;
-    default: hipLaunchKernelGGL((k_probe_mix<4, true, true>), dim3(grid), dim3(kThreads), 0, st, args, nr, nw, nvec, shape, 0x3f803f80u); break;
+    case 1: PCCL_LAUNCH((k_probe_mix<1, true, true>), dim3(grid), dim3(kThreads), 0, st, args, nr, nw, nvec, shape, 0x3f803f80u); break;
+    case 2: PCCL_LAUNCH((k_probe_mix<2, true, true>), dim3(grid), dim3(kThreads), 0, st, args, nr, nw, nvec, shape, 0x3f803f80u); break;
+    default: PCCL_LAUNCH((k_probe_mix<4, true, true>), dim3(grid), dim3(kThreads), 0, st, args, nr, nw, nvec, shape, 0x3f803f80u); break;
   }
   g_launches.fetch_add(1, std::memory_order_relaxed);
   return launch_status(what);

@@ -49,3 +49,6 @@ inline float __uint_as_float(uint32_t u) { float f; std::memcpy(&f, &u, 4); retu
           kernel(__VA_ARGS__);                                           \
         }                                                                \
   } while (0)
+
+// the library's launch macro: no status to collect here
+#define PCCL_LAUNCH(kernel, grid, block, shmem, stream, ...) hipLaunchKernelGGL(kernel, grid, block, shmem, stream, __VA_ARGS__)

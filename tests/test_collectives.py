@@ -517,8 +517,28 @@ def test_repeated_calls_replay_the_checked_arguments(target, mode):
     want = O.ring_reduce_scatter(ins, dtype)
     for r in range(P):
         assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"after set_ rank {r}")
-    # a wrong size is still refused although an entry for these objects exists
+    # a work buffer moved to another storage: the call must use the new one (the old one may be freed memory)
+    if mode != "fused":
+        stale = work[1]
+        stale_bits = stale.clone()
+        work[1] = stale                      # same object ...
+        work[1].set_(torch.full((P * B,), 7.0, device=target.device).untyped_storage(), 0, (P * B,))
+        kept = torch.full((P * B,), 3.0, device=target.device)
+        old_storage_view = kept                # stands in for whatever now owns the old address
+        kernels.reduce_scatter_ranks(t_out, t_in, "ring", mode, work)
+        target.sync()
+        for r in range(P):
+            assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"after work set_ rank {r}")
+        assert not torch.equal(work[1], torch.full((P * B,), 7.0, device=target.device))   # the new storage was used
+        assert torch.equal(old_storage_view, torch.full((P * B,), 3.0, device=target.device))
+    # a wrong size is still refused although an entry for these objects exists: on the first output ...
     t_out[1].set_(torch.zeros(B + 1, device=target.device).untyped_storage(), 0, (B + 1,))
+    with pytest.raises(RuntimeError, match="block_size"):
+        kernels.reduce_scatter_ranks(t_out, t_in, "ring", mode, work)
+    t_out[1].set_(torch.zeros(B, device=target.device).untyped_storage(), 0, (B,))
+    kernels.reduce_scatter_ranks(t_out, t_in, "ring", mode, work)       # an entry for the repaired objects again
+    # ... and on a later one, shrunk in place (same address, fewer elements)
+    t_out[3].resize_(B - 1)
     with pytest.raises(RuntimeError, match="block_size"):
         kernels.reduce_scatter_ranks(t_out, t_in, "ring", mode, work)
     del t_in, t_out, g_out, work, moved
@@ -690,3 +710,110 @@ def test_patch_deepspeed_without_deepspeed_raises(target):
     from pccl import patch_deepspeed as pd
     with pytest.raises(RuntimeError, match="needs the deepspeed package"):
         pd.patch_deepspeed(2, comm=pccl.VirtualWorld(2, target.device).comm(0))
+
+
+# ---------------------------------------------------------------------------
+# buffers that share memory
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("alg,P", [("ring", 5), ("ring", 8), ("recursive", 8), ("recursive", 2)])
+@pytest.mark.parametrize("mode", ["steps", "fused", "faithful"])
+def test_reduce_scatter_in_place(target, dtype, alg, P, mode):
+    """outputs[r] may BE block r of inputs[r] (the reference tolerates it because it
+    copies the input first, pccl/src/reduce_scatter.cpp:119-123): every mode reads
+    an element before the same thread overwrites it."""
+    from pccl import kernels
+    B = 1027
+    ins = make_inputs(P, P * B, dtype, seed=70 + P)
+    t_in = [to_torch(x, dtype, target.device) for x in ins]
+    t_out = [t_in[r][r * B:(r + 1) * B] for r in range(P)]
+    want = (O.ring_reduce_scatter if alg == "ring" else O.recursive_halving_reduce_scatter)(ins, dtype)
+    kernels.reduce_scatter_ranks(t_out, t_in, alg, mode)
+    target.sync()
+    for r in range(P):
+        assert_bits_equal(to_numpy(t_out[r].clone(), dtype), want[r], f"{alg}/{mode} rank {r}")
+        # the other blocks of the input are untouched
+        other = np.delete(to_numpy(t_in[r].clone(), dtype).reshape(P, B), r, axis=0)
+        assert_bits_equal(other.reshape(-1), np.delete(ins[r].reshape(P, B), r, axis=0).reshape(-1), f"rank {r} input")
+
+
+@pytest.mark.parametrize("alg", ["ring", "recursive"])
+@pytest.mark.parametrize("mode", ["steps", "fused"])
+def test_all_gather_in_place(target, alg, mode):
+    """inputs[r] may BE block r of outputs[r] (pccl/src/all_gather.cpp:31-35 copies it there first)."""
+    import torch
+    from pccl import kernels
+    P, n, dtype = 8, 1031, O.F32
+    shards = make_inputs(P, n, dtype, seed=77)
+    t_out = [torch.zeros(P * n, device=target.device) for _ in range(P)]
+    t_in = []
+    for r in range(P):
+        t_out[r][r * n:(r + 1) * n] = to_torch(shards[r], dtype, target.device)
+        t_in.append(t_out[r][r * n:(r + 1) * n])
+    kernels.all_gather_ranks(t_out, t_in, alg, mode)
+    target.sync()
+    for r in range(P):
+        assert_bits_equal(to_numpy(t_out[r], dtype), np.concatenate(shards), f"rank {r}")
+
+
+def test_overlapping_buffers_are_refused(target):
+    """Any other sharing of memory between a written buffer and another buffer of
+    the call is an argument error, reported before anything is launched."""
+    import torch
+    from pccl import kernels
+    P, B = 4, 64
+    dev = target.device
+    t_in = [torch.zeros(P * B, device=dev) for _ in range(P)]
+    t_out = [torch.zeros(B, device=dev) for _ in range(P)]
+    work = [torch.zeros(P * B, device=dev) for _ in range(P)]
+
+    def refused(outs, ins, mode="steps", wk=None, alg="ring"):
+        with pytest.raises(RuntimeError, match="overlap in memory"):
+            kernels.reduce_scatter_ranks(outs, ins, alg, mode, wk)
+
+    # the wrong block of the own input, and another rank's input
+    refused([t_in[0][B:2 * B]] + t_out[1:], t_in, "fused")
+    refused([t_in[1][0:B]] + t_out[1:], t_in, "fused")
+    # the right block, shifted by one element
+    refused([t_in[0][1:B + 1]] + t_out[1:], t_in, "steps", work)
+    # two outputs on the same memory; work space on an input; work space on an output
+    refused([t_out[0], t_out[0]] + t_out[2:], t_in, "fused")
+    refused(t_out, t_in, "steps", [t_in[2]] + work[1:])
+    big = torch.zeros(P * B + B, device=dev)
+    refused([big[P * B - 8:][:B]] + t_out[1:], t_in, "faithful", [big[:P * B]] + work[1:])
+    # inputs may share memory among themselves
+    kernels.reduce_scatter_ranks(t_out, [t_in[0]] * P, "ring", "fused")
+    # all_gather: a shard inside another rank's output, outputs on top of each other
+    g_out = [torch.zeros(P * B, device=dev) for _ in range(P)]
+    g_in = [torch.zeros(B, device=dev) for _ in range(P)]
+    with pytest.raises(RuntimeError, match="overlap in memory"):
+        kernels.all_gather_ranks(g_out, [g_out[1][0:B]] + g_in[1:], "ring", "fused")
+    with pytest.raises(RuntimeError, match="overlap in memory"):
+        kernels.all_gather_ranks([g_out[0], g_out[0]] + g_out[2:], g_in, "recursive", "steps")
+    # the fold: the output on one of its shards; add: a partial overlap
+    sh = [torch.zeros(B, device=dev) for _ in range(3)]
+    with pytest.raises(RuntimeError, match="overlap in memory"):
+        target.native.reduce_kway(sh[1].data_ptr(), [t.data_ptr() for t in sh], B, 0, 0, 0, True, target.stream())
+    with pytest.raises(RuntimeError, match="partly"):
+        target.native.add(big[4:].data_ptr(), big.data_ptr(), sh[0].data_ptr(), B, 0, target.stream())
+    target.sync()
+
+
+def test_fused_ring_beyond_one_launch_refuses_in_place(target):
+    """More ranks than one launch has shard pointers: the chain of launches keeps
+    the running sum in outputs[r] while block r of inputs[r] is still to be added,
+    so in-place use is refused there (the per-step modes take it)."""
+    import torch
+    from pccl import kernels
+    P, B, dtype = 65, 16, O.F32
+    ins = make_inputs(P, P * B, dtype, seed=5)
+    t_in = [to_torch(x, dtype, target.device) for x in ins]
+    t_out = [t_in[r][r * B:(r + 1) * B] for r in range(P)]
+    with pytest.raises(RuntimeError, match="overlap in memory"):
+        kernels.reduce_scatter_ranks(t_out, t_in, "ring", "fused")
+    want = O.ring_reduce_scatter(ins, dtype)
+    kernels.reduce_scatter_ranks(t_out, t_in, "ring", "steps")
+    target.sync()
+    for r in range(P):
+        assert_bits_equal(to_numpy(t_out[r].clone(), dtype), want[r], f"rank {r}")
