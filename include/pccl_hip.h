@@ -266,14 +266,19 @@ int pccl_hip_all_gather_uneven_virtual(void* const* outputs,
  * to [intra, inter, m], reduce-scattered inside the node, then across nodes.
  * The permutation is never materialised: the first inner step reads the inputs
  * through it (strided pieces).  One launch per step serves ALL groups of a
- * level, i.e. (intra-1)+(inter-1) launches for "ring".
+ * level, i.e. (intra-1)+(inter-1) launches for "ring" (one launch per
+ * PCCL_HIP_MAX_RANKS ranks of the grid and step).
  *   inputs[w]  : intra*inter*m elements;  outputs[w] : m elements
  *   work[w]    : intra*inter*m elements (needed if intra > 2 or inter > 2)
  *   mid[w]     : inter*m elements (needed if intra > 1 and inter > 1)
  *   mode       : PCCL_HIP_MODE_STEPS, or PCCL_HIP_MODE_FUSED = ONE launch that
  *                folds all intra*inter inputs in the two-level order
- *                (work and mid may then be NULL).
- * Both levels use `algorithm`; intra*inter <= PCCL_HIP_MAX_RANKS. */
+ *                (work and mid may then be NULL).  A grid of more than
+ *                PCCL_HIP_MAX_RANKS ranks is fused level by level instead: one
+ *                fold per node over its `intra` inputs into mid[] (which is
+ *                then needed; work is not), then one fold per local rank over
+ *                the `inter` intermediates; intra, inter <= PCCL_HIP_MAX_RANKS.
+ * Both levels use `algorithm`; intra*inter <= PCCL_HIP_MAX_VIRTUAL_RANKS. */
 int pccl_hip_reduce_scatter_2d_virtual(void* const* outputs,
                                        const void* const* inputs,
                                        void* const* work, void* const* mid,
@@ -286,7 +291,8 @@ int pccl_hip_reduce_scatter_2d_virtual(void* const* outputs,
  * stage writes through the un-permutation, so no extra pass is made.
  *   inputs[w]  : block_bytes bytes;  outputs[w] : intra*inter*block_bytes
  *   mid[w]     : inter*block_bytes bytes (needed if intra > 1 and inter > 1)
- * PCCL_HIP_MODE_FUSED places every shard directly (one launch). */
+ * PCCL_HIP_MODE_FUSED places every shard directly (one launch per 64 shards
+ * and 64 outputs).  intra*inter <= PCCL_HIP_MAX_VIRTUAL_RANKS. */
 int pccl_hip_all_gather_2d_virtual(void* const* outputs,
                                    const void* const* inputs, void* const* mid,
                                    int intra, int inter, size_t block_bytes,

@@ -1455,32 +1455,41 @@ int pccl_hip_reduce_scatter_2d_virtual(void* const* outputs, const void* const* 
   const bool rec = !strcmp(algorithm, "recursive");
   if (!ring && !rec)
     return fail(PCCL_HIP_EINVAL, "Unknown algorithm specified for reduce_scatter_mpi: %s", algorithm);
-  if (intra < 1 || inter < 1 || (long)intra * inter > kMaxSeg)
+  if (intra < 1 || inter < 1 || (long)intra * inter > kMaxVirtualRanks)
     return fail(PCCL_HIP_EINVAL, "%s: intra = %d, inter = %d: need intra, inter >= 1 and intra*inter <= %d",
-                what, intra, inter, kMaxSeg);
+                what, intra, inter, kMaxVirtualRanks);
   if (rec && (!pow2(intra) || !pow2(inter)))
     return fail(PCCL_HIP_EINVAL, "%s: recursive halving needs power-of-two group sizes, got %d x %d", what,
                 intra, inter);
   if (mode != PCCL_HIP_MODE_STEPS && mode != PCCL_HIP_MODE_FUSED)
     return fail(PCCL_HIP_EINVAL, "%s: mode %d not offered here (steps or fused)", what, mode);
   const int W = intra * inter;
+  // a grid beyond the shards of one launch is fused level by level: one fold per node, then one per local rank
+  const bool fused = mode == PCCL_HIP_MODE_FUSED;
+  const bool two_folds = fused && W > kMaxSeg;
+  if (two_folds && (intra > kMaxSeg || inter > kMaxSeg))
+    return fail(PCCL_HIP_EINVAL, "%s: the fused mode takes groups of at most %d ranks per level, got %d x %d (use the per-step mode)",
+                what, kMaxSeg, intra, inter);
   if (int rc = check_table((const void* const*)outputs, W, what, "outputs")) return rc;
   if (int rc = check_table(inputs, W, what, "inputs")) return rc;
+  const bool need_mid = (!fused || two_folds) && intra > 1 && inter > 1;
+  const bool need_work = !fused && (intra > 2 || inter > 2);
+  if (need_mid) if (int rc = check_table((const void* const*)mid, W, what, "mid")) return rc;
+  if (need_work) if (int rc = check_table((const void* const*)work, W, what, "work")) return rc;
   if (m == 0) return PCCL_HIP_OK;
   hipStream_t st = (hipStream_t)stream;
   const size_t es = esize_of(dtype);
   {
-    const bool steps = mode == PCCL_HIP_MODE_STEPS;
     ExtentList ext;
     for (int w = 0; w < W; ++w) ext.add(inputs[w], (size_t)W * m * es, w, 'i');
     for (int w = 0; w < W; ++w)
       ext.add(outputs[w], m * es, w, 'o', outputs[w] == (const uint8_t*)inputs[w] + (size_t)w * m * es);
-    if (steps && (intra > 2 || inter > 2) && work) for (int w = 0; w < W; ++w) ext.add(work[w], (size_t)W * m * es, w, 'w');
-    if (steps && intra > 1 && inter > 1 && mid) for (int w = 0; w < W; ++w) ext.add(mid[w], (size_t)inter * m * es, w, 'w');
+    if (need_work) for (int w = 0; w < W; ++w) ext.add(work[w], (size_t)W * m * es, w, 'w');
+    if (need_mid) for (int w = 0; w < W; ++w) ext.add(mid[w], (size_t)inter * m * es, w, 'w');
     if (int rc = ext.check(what)) return rc;
   }
   // inputs of W*m elements per rank, as much work space in the per-step mode, the outputs
-  CallBytes footprint(((mode == PCCL_HIP_MODE_FUSED ? 1 : 2) * (size_t)W * W + W) * m * es);
+  CallBytes footprint(((fused ? 1 : 2) * (size_t)W * W + W) * m * es);
   auto at = [es](const void* p, size_t elems) { return (const void*)((const uint8_t*)p + elems * es); };
   auto atw = [es](void* p, size_t elems) { return (void*)((uint8_t*)p + elems * es); };
 
@@ -1490,7 +1499,7 @@ int pccl_hip_reduce_scatter_2d_virtual(void* const* outputs, const void* const* 
     return launch_copy(c, 1, st, what);
   }
 
-  if (mode == PCCL_HIP_MODE_FUSED) {
+  if (fused && !two_folds) {
     KwayArgs args;
     if (ring) {
       // world order; block w of every input; inner ring inside each node, then the ring across nodes
@@ -1507,44 +1516,85 @@ int pccl_hip_reduce_scatter_2d_virtual(void* const* outputs, const void* const* 
     return launch_kway(args, W, W, W, m, dtype, PCCL_HIP_ORDER_HALVING, 0, 1, st, what);
   }
 
-  const bool need_mid = intra > 1 && inter > 1;
-  const bool need_work = intra > 2 || inter > 2;
-  if (need_mid) if (int rc = check_table((const void* const*)mid, W, what, "mid")) return rc;
-  if (need_work) if (int rc = check_table((const void* const*)work, W, what, "work")) return rc;
   // result of the inner stage: [inter, m] per rank
-  const void* midr[kMaxSeg];
-  void* midw[kMaxSeg];
+  RankList<const void*> midr((size_t)W);
+  RankList<void*> midw((size_t)W);
   for (int w = 0; w < W; ++w) {
     if (intra == 1) { midr[w] = inputs[w]; midw[w] = nullptr; }
     else if (inter == 1) { midr[w] = outputs[w]; midw[w] = outputs[w]; }
     else { midr[w] = mid[w]; midw[w] = mid[w]; }
   }
   const size_t B1 = (size_t)inter * m;   // inner block: one piece of m per node
+  const int order = ring ? PCCL_HIP_ORDER_RING : PCCL_HIP_ORDER_HALVING;
+
+  if (two_folds) {
+    // Inner level, node by node: element (jj, i) of rank (j, i)'s intermediate is the fold, in the inner
+    // schedule's order for local rank i, of block jj*intra + i of the node's `intra` inputs.  The outputs of
+    // a launch are taken in the order o = jj*intra + i, whole rows of `intra` at a time, so that output o of
+    // a launch starts its schedule at shard (first0 + o) mod intra as the flat collective does.
+    if (intra > 1) {
+      const int rows_per = kMaxSeg / intra;   // rows jj of one launch
+      for (int j = 0; j < inter; ++j)
+        for (int jj0 = 0; jj0 < inter; jj0 += rows_per) {
+          const int rows = inter - jj0 < rows_per ? inter - jj0 : rows_per;
+          KwayArgs args;
+          for (int i = 0; i < intra; ++i) args.shard[i] = inputs[j * intra + i];
+          for (int r = 0; r < rows; ++r)
+            for (int i = 0; i < intra; ++i) {
+              const int o = r * intra + i, jj = jj0 + r;
+              args.out[o] = atw(midw[j * intra + i], (size_t)jj * m);
+              args.eoff[o] = (size_t)(jj * intra + i) * m;
+            }
+          if (int rc = launch_kway(args, intra, intra, rows * intra, m, dtype, order, ring ? 1 : 0, 1, st, what)) return rc;
+        }
+    }
+    // Outer level, local rank by local rank: a flat fused reduce_scatter over the `inter` intermediates.
+    if (inter > 1) {
+      for (int i = 0; i < intra; ++i) {
+        KwayArgs args;
+        for (int j = 0; j < inter; ++j) {
+          args.shard[j] = midr[j * intra + i]; args.out[j] = outputs[j * intra + i]; args.eoff[j] = (size_t)j * m;
+        }
+        if (int rc = launch_kway(args, inter, inter, inter, m, dtype, order, ring ? 1 : 0, 1, st, what)) return rc;
+      }
+    }
+    return PCCL_HIP_OK;
+  }
+
+  // per-step mode: one step of a level for ALL its groups is one launch per kMaxSeg ranks
+  RankList<AddTriple> adds((size_t)W);
+  auto launch_step = [&](const Pieces& pc) {
+    for (int w0 = 0; w0 < W; w0 += kMaxSeg) {
+      const int cnt = W - w0 < kMaxSeg ? W - w0 : kMaxSeg;
+      AddSegs segs;
+      for (int q = 0; q < cnt; ++q) { segs.dst[q] = adds[w0 + q].dst; segs.a[q] = adds[w0 + q].a; segs.b[q] = adds[w0 + q].b; }
+      if (int rc = launch_add_pieces(segs, cnt, pc, dtype, st, what)) return rc;
+    }
+    return (int)PCCL_HIP_OK;
+  };
 
   // ---- inner stage: groups of `intra` ranks, inputs read through the permutation ----
   if (intra > 1 && ring) {
     for (int s = 0; s < intra - 1; ++s) {
-      AddSegs segs;
       const bool first = s == 0, last = s == intra - 2;
       for (int j = 0; j < inter; ++j)
         for (int i = 0; i < intra; ++i) {
           const int w = j * intra + i;
           const int b = ((i - s - 2) % intra + intra) % intra;
           const int src = j * intra + (i - 1 + intra) % intra;
-          segs.a[w] = at(inputs[w], (size_t)b * m);
-          segs.b[w] = first ? at(inputs[src], (size_t)b * m) : at(work[src], (size_t)b * B1);
-          segs.dst[w] = last ? midw[w] : atw(work[w], (size_t)b * B1);
+          adds[w].a = at(inputs[w], (size_t)b * m);
+          adds[w].b = first ? at(inputs[src], (size_t)b * m) : at(work[src], (size_t)b * B1);
+          adds[w].dst = last ? midw[w] : atw(work[w], (size_t)b * B1);
         }
       Pieces pc{};
       pc.s1 = (unsigned)inter; pc.s2 = 1; pc.len = m;
       pc.a1 = (size_t)intra * m; pc.b1 = first ? (size_t)intra * m : m; pc.d1 = m;
-      if (int rc = launch_add_pieces(segs, W, pc, dtype, st, what)) return rc;
+      if (int rc = launch_step(pc)) return rc;
     }
   } else if (intra > 1) {
     int rounds = 0;
     while ((1 << rounds) < intra) ++rounds;
     for (int t = 0; t < rounds; ++t) {
-      AddSegs segs;
       const int g = intra >> t, half = g / 2;
       const bool first = t == 0, last = t == rounds - 1;
       for (int j = 0; j < inter; ++j)
@@ -1554,13 +1604,13 @@ int pccl_hip_reduce_scatter_2d_virtual(void* const* outputs, const void* const* 
           const int p = j * intra + (lower ? i + half : i - half);
           const size_t b0 = (size_t)(i / g) * g + (lower ? 0 : half);   // first block this rank keeps
           if (first) {
-            segs.a[w] = at(inputs[w], b0 * m);
-            segs.b[w] = at(inputs[p], b0 * m);
+            adds[w].a = at(inputs[w], b0 * m);
+            adds[w].b = at(inputs[p], b0 * m);
           } else {
-            segs.a[w] = at(work[w], b0 * B1);
-            segs.b[w] = at(work[p], b0 * B1);
+            adds[w].a = at(work[w], b0 * B1);
+            adds[w].b = at(work[p], b0 * B1);
           }
-          segs.dst[w] = last ? midw[w] : atw(work[w], b0 * B1);
+          adds[w].dst = last ? midw[w] : atw(work[w], b0 * B1);
         }
       Pieces pc{};
       if (first) {   // piece (node jj, block bb): strided in the input, contiguous rows in the work layout
@@ -1570,31 +1620,29 @@ int pccl_hip_reduce_scatter_2d_virtual(void* const* outputs, const void* const* 
       } else {
         pc = contiguous((size_t)half * B1);
       }
-      if (int rc = launch_add_pieces(segs, W, pc, dtype, st, what)) return rc;
+      if (int rc = launch_step(pc)) return rc;
     }
   }
 
   // ---- outer stage: groups of `inter` ranks on the [inter, m] intermediates ----
   if (inter > 1 && ring) {
     for (int s = 0; s < inter - 1; ++s) {
-      AddSegs segs;
       const bool first = s == 0, last = s == inter - 2;
       for (int j = 0; j < inter; ++j)
         for (int i = 0; i < intra; ++i) {
           const int w = j * intra + i;
           const int b = ((j - s - 2) % inter + inter) % inter;
           const int src = ((j - 1 + inter) % inter) * intra + i;
-          segs.a[w] = at(midr[w], (size_t)b * m);
-          segs.b[w] = first ? at(midr[src], (size_t)b * m) : at(work[src], (size_t)b * m);
-          segs.dst[w] = last ? outputs[w] : atw(work[w], (size_t)b * m);
+          adds[w].a = at(midr[w], (size_t)b * m);
+          adds[w].b = first ? at(midr[src], (size_t)b * m) : at(work[src], (size_t)b * m);
+          adds[w].dst = last ? outputs[w] : atw(work[w], (size_t)b * m);
         }
-      if (int rc = launch_add(segs, W, m, dtype, st, what)) return rc;
+      if (int rc = launch_step(contiguous(m))) return rc;
     }
   } else if (inter > 1) {
     int rounds = 0;
     while ((1 << rounds) < inter) ++rounds;
     for (int t = 0; t < rounds; ++t) {
-      AddSegs segs;
       const int g = inter >> t, half = g / 2;
       const bool first = t == 0, last = t == rounds - 1;
       for (int j = 0; j < inter; ++j)
@@ -1603,11 +1651,11 @@ int pccl_hip_reduce_scatter_2d_virtual(void* const* outputs, const void* const* 
           const bool lower = (j % g) < half;
           const int p = (lower ? j + half : j - half) * intra + i;
           const size_t b0 = (size_t)(j / g) * g + (lower ? 0 : half);
-          segs.a[w] = first ? at(midr[w], b0 * m) : at(work[w], b0 * m);
-          segs.b[w] = first ? at(midr[p], b0 * m) : at(work[p], b0 * m);
-          segs.dst[w] = last ? outputs[w] : atw(work[w], b0 * m);
+          adds[w].a = first ? at(midr[w], b0 * m) : at(work[w], b0 * m);
+          adds[w].b = first ? at(midr[p], b0 * m) : at(work[p], b0 * m);
+          adds[w].dst = last ? outputs[w] : atw(work[w], b0 * m);
         }
-      if (int rc = launch_add(segs, W, (size_t)half * m, dtype, st, what)) return rc;
+      if (int rc = launch_step(contiguous((size_t)half * m))) return rc;
     }
   }
   return PCCL_HIP_OK;
@@ -1622,9 +1670,9 @@ int pccl_hip_all_gather_2d_virtual(void* const* outputs, const void* const* inpu
   const bool rec = !strcmp(algorithm, "recursive");
   if (!ring && !rec)
     return fail(PCCL_HIP_EINVAL, "Unknown algorithm specified for all_gather_mpi: %s", algorithm);
-  if (intra < 1 || inter < 1 || (long)intra * inter > kMaxSeg)
+  if (intra < 1 || inter < 1 || (long)intra * inter > kMaxVirtualRanks)
     return fail(PCCL_HIP_EINVAL, "%s: intra = %d, inter = %d: need intra, inter >= 1 and intra*inter <= %d",
-                what, intra, inter, kMaxSeg);
+                what, intra, inter, kMaxVirtualRanks);
   if (rec && (!pow2(intra) || !pow2(inter)))
     return fail(PCCL_HIP_EINVAL, "%s: recursive doubling needs power-of-two group sizes, got %d x %d", what,
                 intra, inter);
@@ -1653,24 +1701,35 @@ int pccl_hip_all_gather_2d_virtual(void* const* outputs, const void* const* inpu
   }
 
   if (mode == PCCL_HIP_MODE_FUSED) {   // the 2-D result is the concatenation in world order
-    size_t nbytes[kMaxSeg], off[kMaxSeg];
+    RankList<size_t> nbytes((size_t)W), off((size_t)W);
     for (int w = 0; w < W; ++w) { nbytes[w] = n; off[w] = (size_t)w * n; }
-    return pccl_hip_all_gather_uneven_virtual(outputs, inputs, nbytes, off, W, stream);
+    return pccl_hip_all_gather_uneven_virtual(outputs, inputs, &nbytes[0], &off[0], W, stream);
   }
 
   const bool need_mid = intra > 1 && inter > 1;
   if (need_mid) if (int rc = check_table((const void* const*)mid, W, what, "mid")) return rc;
   // outer result per rank, [inter, n]; with one rank per node it IS the output
-  uint8_t* M[kMaxSeg];
+  RankList<uint8_t*> M((size_t)W);
   for (int w = 0; w < W; ++w)
     M[w] = inter == 1 ? (uint8_t*)inputs[w] : intra == 1 ? (uint8_t*)outputs[w] : (uint8_t*)mid[w];
-  CopyPairs c;
+  // one step of a level for ALL its groups: one launch per kMaxSeg ranks
+  struct Pair { void* dst; const void* src; };
+  RankList<Pair> c((size_t)W);
+  auto launch_step = [&](const Pieces& pieces) {
+    for (int w0 = 0; w0 < W; w0 += kMaxSeg) {
+      const int cnt = W - w0 < kMaxSeg ? W - w0 : kMaxSeg;
+      CopyPairs cp;
+      for (int q = 0; q < cnt; ++q) { cp.dst[q] = c[w0 + q].dst; cp.src[q] = c[w0 + q].src; }
+      if (int rc = launch_copy_pieces(cp, cnt, pieces, st, what)) return rc;
+    }
+    return (int)PCCL_HIP_OK;
+  };
 
   // ---- outer stage: gather across nodes into M ----
   if (inter > 1) {
     for (int j = 0; j < inter; ++j)
-      for (int i = 0; i < intra; ++i) { const int w = j * intra + i; c.dst[w] = M[w] + (size_t)j * n; c.src[w] = inputs[w]; }
-    if (int rc = launch_copy_pieces(c, W, contiguous(n), st, what)) return rc;
+      for (int i = 0; i < intra; ++i) { const int w = j * intra + i; c[w].dst = M[w] + (size_t)j * n; c[w].src = inputs[w]; }
+    if (int rc = launch_step(contiguous(n))) return rc;
     if (rec) {
       for (int seg = 1; seg < inter; seg *= 2) {
         for (int j = 0; j < inter; ++j)
@@ -1678,9 +1737,9 @@ int pccl_hip_all_gather_2d_virtual(void* const* outputs, const void* const* inpu
             const int w = j * intra + i, pj = j ^ seg, p = pj * intra + i;
             const int gs = (j / (2 * seg)) * (2 * seg);
             const size_t off = (size_t)(j < pj ? gs + seg : gs) * n;
-            c.dst[w] = M[w] + off; c.src[w] = M[p] + off;
+            c[w].dst = M[w] + off; c[w].src = M[p] + off;
           }
-        if (int rc = launch_copy_pieces(c, W, contiguous((size_t)seg * n), st, what)) return rc;
+        if (int rc = launch_step(contiguous((size_t)seg * n))) return rc;
       }
     } else {
       for (int s = 0; s < inter - 1; ++s) {
@@ -1688,9 +1747,9 @@ int pccl_hip_all_gather_2d_virtual(void* const* outputs, const void* const* inpu
           for (int i = 0; i < intra; ++i) {
             const int w = j * intra + i, src = ((j - 1 + inter) % inter) * intra + i;
             const size_t off = (size_t)(((j - s - 1) % inter + inter) % inter) * n;
-            c.dst[w] = M[w] + off; c.src[w] = M[src] + off;
+            c[w].dst = M[w] + off; c[w].src = M[src] + off;
           }
-        if (int rc = launch_copy_pieces(c, W, contiguous(n), st, what)) return rc;
+        if (int rc = launch_step(contiguous(n))) return rc;
       }
     }
   }
@@ -1701,8 +1760,8 @@ int pccl_hip_all_gather_2d_virtual(void* const* outputs, const void* const* inpu
   Pieces pc{};
   pc.s1 = (unsigned)inter; pc.s2 = 1; pc.len = n; pc.d1 = (size_t)intra * n; pc.a1 = n;
   for (int j = 0; j < inter; ++j)
-    for (int i = 0; i < intra; ++i) { const int w = j * intra + i; c.dst[w] = (uint8_t*)outputs[w] + (size_t)i * n; c.src[w] = M[w]; }
-  if (int rc = launch_copy_pieces(c, W, pc, st, what)) return rc;
+    for (int i = 0; i < intra; ++i) { const int w = j * intra + i; c[w].dst = (uint8_t*)outputs[w] + (size_t)i * n; c[w].src = M[w]; }
+  if (int rc = launch_step(pc)) return rc;
   pc.a1 = (size_t)intra * n;   // from here on both sides are output layouts
   if (rec) {
     for (int seg = 1; seg < intra; seg *= 2) {
@@ -1711,10 +1770,10 @@ int pccl_hip_all_gather_2d_virtual(void* const* outputs, const void* const* inpu
           const int w = j * intra + i, pi = i ^ seg, p = j * intra + pi;
           const int gs = (i / (2 * seg)) * (2 * seg);
           const size_t off = (size_t)(i < pi ? gs + seg : gs) * n;
-          c.dst[w] = (uint8_t*)outputs[w] + off; c.src[w] = (const uint8_t*)outputs[p] + off;
+          c[w].dst = (uint8_t*)outputs[w] + off; c[w].src = (const uint8_t*)outputs[p] + off;
         }
       pc.len = (size_t)seg * n;
-      if (int rc = launch_copy_pieces(c, W, pc, st, what)) return rc;
+      if (int rc = launch_step(pc)) return rc;
     }
   } else {
     for (int s = 0; s < intra - 1; ++s) {
@@ -1722,10 +1781,10 @@ int pccl_hip_all_gather_2d_virtual(void* const* outputs, const void* const* inpu
         for (int i = 0; i < intra; ++i) {
           const int w = j * intra + i, src = j * intra + (i - 1 + intra) % intra;
           const size_t off = (size_t)(((i - s - 1) % intra + intra) % intra) * n;
-          c.dst[w] = (uint8_t*)outputs[w] + off; c.src[w] = (const uint8_t*)outputs[src] + off;
+          c[w].dst = (uint8_t*)outputs[w] + off; c[w].src = (const uint8_t*)outputs[src] + off;
         }
       pc.len = n;
-      if (int rc = launch_copy_pieces(c, W, pc, st, what)) return rc;
+      if (int rc = launch_step(pc)) return rc;
     }
   }
   return PCCL_HIP_OK;

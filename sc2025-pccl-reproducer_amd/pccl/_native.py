@@ -25,7 +25,7 @@ MODE_STEPS = 0
 MODE_FUSED = 1
 MODE_FAITHFUL = 2
 
-MAX_RANKS = 64            # per launch / fused modes / 2-D grids
+MAX_RANKS = 64            # segments / shards of one launch
 MAX_VIRTUAL_RANKS = 4096  # per-step modes of the 1-D collectives
 NOALLOC_SCRATCH_BYTES = 32 << 20   # built-in work space of reduce_scatter_virtual_noalloc
 ABI_VERSION = 1

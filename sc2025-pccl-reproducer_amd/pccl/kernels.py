@@ -469,8 +469,8 @@ def _check_2d(outputs, inputs, intra, inter):
     W = intra * inter
     if intra < 1 or inter < 1 or len(inputs) != W or len(outputs) != W:
         raise ValueError("need intra*inter inputs and outputs, in world-rank order")
-    if W > MAX_RANKS:
-        raise RuntimeError(f"at most {MAX_RANKS} virtual ranks per 2-D grid")
+    if W > MAX_VIRTUAL_RANKS:
+        raise RuntimeError(f"at most {MAX_VIRTUAL_RANKS} virtual ranks per 2-D grid")
     for t in inputs:
         check_device_tensor(t, "input")
     for t in outputs:
@@ -499,11 +499,14 @@ def reduce_scatter_2d_ranks(outputs: Sequence[torch.Tensor], inputs: Sequence[to
     if code == MODE_FAITHFUL:
         code = MODE_STEPS
     work = mid = None
-    if code == MODE_STEPS:
-        if intra > 2 or inter > 2:
-            work = [torch.empty_like(inputs[w]) for w in range(W)]
-        if intra > 1 and inter > 1:
-            mid = [torch.empty(inter * m, dtype=dt, device=inputs[0].device) for _ in range(W)]
+    if code == MODE_FUSED and W > MAX_RANKS and max(intra, inter) > MAX_RANKS:
+        code = MODE_STEPS                 # the fused mode folds at most MAX_RANKS ranks per level; same bits step by step
+    if code == MODE_STEPS and (intra > 2 or inter > 2):
+        work = [torch.empty_like(inputs[w]) for w in range(W)]
+    # the intermediates between the levels: the per-step mode, and the fused mode beyond the shards of one
+    # launch (one fold per node, then one per local rank)
+    if (code == MODE_STEPS or W > MAX_RANKS) and intra > 1 and inter > 1:
+        mid = [torch.empty(inter * m, dtype=dt, device=inputs[0].device) for _ in range(W)]
     _native.load().reduce_scatter_2d_virtual(_ptrs(outputs), _ptrs(inputs), _ptrs(work), _ptrs(mid), intra, inter,
                                              m, dtype_code(dt), algorithm, code, stream_handle())
 

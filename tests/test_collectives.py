@@ -376,7 +376,9 @@ def test_all_gather_2D(target, intra, inter, use_rd, cpp):
         assert torch.equal(t_out[r], cat)      # the 2-D all_gather is a plain concatenation
 
 
-GRIDS = [(1, 1), (2, 1), (1, 2), (2, 2), (4, 2), (2, 4), (3, 2), (2, 3), (1, 8), (8, 1), (4, 4), (8, 8), (16, 4)]
+# the last row: more ranks than one launch has pointers for (steps: launches of 64 ranks; fused: level by level)
+GRIDS = [(1, 1), (2, 1), (1, 2), (2, 2), (4, 2), (2, 4), (3, 2), (2, 3), (1, 8), (8, 1), (4, 4), (8, 8), (16, 4),
+         (8, 16), (16, 16), (5, 13), (43, 3), (1, 128), (128, 1)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -391,7 +393,7 @@ def test_reduce_scatter_2d_driver(target, dtype, intra, inter, alg, mode):
     if alg == "recursive" and ((intra & (intra - 1)) or (inter & (inter - 1))):
         pytest.skip("halving needs power-of-two groups")
     W = intra * inter
-    m = 261 if W <= 16 else 37
+    m = 261 if W <= 16 else 37 if W <= 64 else 13
     print(f"reduce_scatter_2d {intra}x{inter} alg={alg} mode={mode} dtype={dtype}", flush=True)
     ins = make_inputs(W, W * m, dtype, seed=61)
     t_in = [to_torch(x, dtype, target.device) for x in ins]
@@ -413,7 +415,7 @@ def test_all_gather_2d_driver(target, intra, inter, alg, mode):
     if alg == "recursive" and ((intra & (intra - 1)) or (inter & (inter - 1))):
         pytest.skip("doubling needs power-of-two groups")
     W = intra * inter
-    n = 1030 if W <= 16 else 70
+    n = 1030 if W <= 16 else 70 if W <= 64 else 22
     rng = np.random.default_rng(71)
     ins = [rng.integers(0, 256, n, dtype=np.uint8) for _ in range(W)]
     t_in = [torch.from_numpy(x).to(target.device) for x in ins]
