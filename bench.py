@@ -219,7 +219,7 @@ def make_ring_rs(P, elems_per_rank, dtype, modes, device, seed=1234, std=1.0):
         else:
             kernel_bytes = 3 * P * B * es                   # one batched step: 2 reads + 1 write per rank
             alg_bytes = (P - 1) * kernel_bytes
-            kernel = "k_add_segs"
+            kernel = "k_add_rows"
         out[mode] = (step, dict(
             alg_bytes=alg_bytes, kernel=kernel, kernel_bytes=kernel_bytes,
             kernel_launches=(P - 1 if m != kernels.MODE_FUSED else 1), launches=launches,
@@ -260,7 +260,7 @@ def make_rh_pair(count_elems, device, seed=7):
         return True
 
     kb = 2 * 3 * B * 2
-    info = dict(alg_bytes=kb, kernel="k_rh_round", kernel_bytes=kb, kernel_launches=1, launches=1,
+    info = dict(alg_bytes=kb, kernel="k_rh_rows", kernel_bytes=kb, kernel_launches=1, launches=1,
                 desc=f"recursive-halving round, one pair of ranks, bf16, halves of {B * 2 / MiB:.0f} MiB "
                      f"(round 0 of P=64 with {4 * B / MiB:.0f} MiB per rank)",
                 dtype="bf16", P=2, B=B, verify=verify,
@@ -312,7 +312,7 @@ def make_rh_full(P, elems_per_rank, modes, device, seed=21):
         else:
             # round r adds (P / 2^(r+1)) blocks per rank: 2 reads + 1 write per element
             alg = sum(3 * P * (P >> (r + 1)) * B * 2 for r in range(rounds))
-            kb, kernel, kl, launches = alg, "k_rh_round", 1, rounds
+            kb, kernel, kl, launches = alg, "k_rh_rows", 1, rounds
         out[mode] = (step, dict(
             alg_bytes=alg, kernel=kernel, kernel_bytes=kb, kernel_launches=kl, launches=launches,
             desc=f"recursive-halving reduce_scatter, P={P} resident virtual ranks, bf16, {total} elements per "
@@ -424,7 +424,7 @@ def make_kway(k, n, modes, device, seed=11):
         per_hop = kernels.mode_code(mode if mode else "fused") != kernels.MODE_FUSED
         if per_hop:
             kb = 3 * n * 4                                       # one hop: 2 reads + 1 write
-            info = dict(alg_bytes=(k - 1) * kb, kernel="k_add_segs", kernel_bytes=kb, kernel_launches=k - 1,
+            info = dict(alg_bytes=(k - 1) * kb, kernel="k_add_rows", kernel_bytes=kb, kernel_launches=k - 1,
                         launches=k - 1,
                         desc=f"reduce of {k} fp32 shards of {n} elements ({n * 4 / MiB:.0f} MiB each) as {k - 1} "
                              f"per-hop accumulate launches, ring order", dtype="f32", P=k, B=n, verify=verify)
@@ -615,7 +615,7 @@ def ceilings(steps, warmup, device):
                 if v > best:
                     best, shape = v, f"shape {sh}, {u} vectors per thread"
         if nw == 1 and nr == 2:
-            mine, kname = gbps(lambda: kernels.add(wr[0], rd[0], rd[1]), 3 * nb), "k_add_segs"
+            mine, kname = gbps(lambda: kernels.add(wr[0], rd[0], rd[1]), 3 * nb), "k_add_rows"
         elif nw == 1:
             mine, kname = gbps(lambda: kernels.reduce_kway(wr[0], rd, "ring", 1), (nr + 1) * nb), "k_reduce_kway"
         else:
@@ -811,24 +811,90 @@ def drop_in(device, steps=5, warmup=2):
 # CPU baseline (oracle/cpu_baseline.c), bounded sample
 # ---------------------------------------------------------------------------
 
-def cpu_baseline(info):
-    """Time the reference's per-rank ring reduce_scatter on host cores for a
-    bounded sample of the workload (same P and dtype, shorter blocks)."""
+def _run_reaped(cmd, timeout):
+    """Run a launcher in a process group of its own and leave nothing of it behind:
+    an MPI launcher returns before its proxies have gone, so the group is waited
+    for (two seconds at most) and then ended."""
+    import signal
+    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, start_new_session=True)
+    try:
+        out, _ = proc.communicate(timeout=timeout)
+        rc = proc.returncode
+    except subprocess.TimeoutExpired:
+        out, rc = "", -1
+    pgid = proc.pid                      # the session leader's pid is the group's id
+    deadline = time.time() + 2.0
+    while True:
+        try:
+            os.killpg(pgid, 0)
+        except (ProcessLookupError, PermissionError):
+            break                        # nobody left in the group
+        if time.time() > deadline:
+            try:
+                os.killpg(pgid, signal.SIGKILL)
+            except (ProcessLookupError, PermissionError):
+                pass
+            break
+        time.sleep(0.02)
+    if proc.poll() is None:
+        proc.wait()
+    return rc, out
+
+
+def _cpu_leg(ranks, dtype, block, iters, algs, scale):
+    """One shape of the per-rank CPU program for the algorithms in `algs`
+    ('ring': the reference's ring over MPI_Sendrecv, pccl/src/reduce_scatter.cpp:101-155;
+    'mpi_block': MPI_Reduce_scatter_block, what pccl/reduce_scatter.py:197 calls).
+    Returns {alg: result of the program}, the transport used and the wall seconds."""
     build = os.path.join(ROOT, "oracle", "build")
     mpi_bin = os.path.join(build, "cpu_baseline_mpi")
     shm_bin = os.path.join(build, "cpu_baseline_shm")
-    if not os.path.exists(shm_bin):
+    launcher = None
+    for cand in ("/opt/conda/bin/mpiexec.hydra", shutil.which("mpiexec.hydra"), shutil.which("mpiexec")):
+        if cand and os.path.exists(cand):
+            launcher = cand
+            break
+    res, transport, t0 = {}, None, time.time()
+    for alg in algs:
+        args = ["--alg", alg, "--dtype", dtype, "--block", str(block), "--warmup", "1", "--iters", str(iters),
+                "--scale", scale]
+        attempts = []
+        if launcher and os.path.exists(mpi_bin):
+            attempts.append(([launcher, "-np", str(ranks), mpi_bin] + args, "MPI_Sendrecv (MPICH)"))
+        if alg == "ring":                # the vendor collective exists over MPI only
+            attempts.append(([shm_bin, "--ranks", str(ranks)] + args, "fork+shared memory"))
+        for cmd, how in attempts:
+            try:
+                rc, out = _run_reaped(cmd, 400)
+            except Exception:                                 # noqa: BLE001
+                continue
+            line = [l for l in out.splitlines() if l.startswith("{")]
+            if rc == 0 and line:
+                res[alg] = json.loads(line[-1])
+                transport = transport or how
+                break
+    return res, transport, time.time() - t0
+
+
+def cpu_baseline(info):
+    """The reference's per-rank algorithms on the host cores (oracle/cpu_baseline.c),
+    timed on bounded samples: the headline's own shape (ring reduce_scatter over
+    MPI_Sendrecv), and the reference's CPU-runnable configuration -- ring
+    reduce_scatter, P = 4, fp32, 16 Mi elements per rank -- both as the
+    hand-written ring and as the vendor's MPI_Reduce_scatter_block."""
+    build = os.path.join(ROOT, "oracle", "build")
+    if not os.path.exists(os.path.join(build, "cpu_baseline_shm")):
         try:
             subprocess.run(["make", "-C", os.path.join(ROOT, "oracle")], check=True, capture_output=True)
         except Exception as e:                               # noqa: BLE001
             return {"value": None, "unit": "GB/s", "cores": 0, "kind": "port", "sample": f"not built: {e}"}
-    P = info["P"] if info["kernel"] in ("k_add_segs", "k_reduce_kway") and info["P"] <= 8 else 8
+    P = info["P"] if info["kernel"] in ("k_add_rows", "k_add_segs", "k_reduce_kway") and info["P"] <= 8 else 8
     dtype = "bf16" if info["dtype"] == "bf16" else "f32"
     host_cores = os.cpu_count() or 1
     ranks = min(P, max(1, host_cores))
     if ranks & (ranks - 1):
         ranks = 1 << (ranks.bit_length() - 1)
-    if info["kernel"] == "k_add_segs" and ranks == info["P"]:
+    if info["kernel"] in ("k_add_rows", "k_add_segs") and ranks == info["P"]:
         block, sample = info["B"], "the workload itself (same P, dtype and block size)"
     else:
         block = (1 << 22) if dtype == "bf16" else (1 << 21)                 # 8 MiB blocks
@@ -836,47 +902,30 @@ def cpu_baseline(info):
     # about ten seconds of timed calls, assuming ~15 GB/s of algorithmic bytes on the host
     job_bytes = 3 * (ranks - 1) * block * (2 if dtype == "bf16" else 4) * ranks
     iters = max(5, min(500, int(10.0 / max(job_bytes / 15e9, 1e-3))))
-    args = ["--alg", "ring", "--dtype", dtype, "--block", str(block), "--warmup", "1", "--iters", str(iters),
-            "--scale", "0.01" if dtype == "bf16" else "1.0"]
-    launcher = None
-    for cand in ("/opt/conda/bin/mpiexec.hydra", shutil.which("mpiexec.hydra"), shutil.which("mpiexec")):
-        if cand and os.path.exists(cand):
-            launcher = cand
-            break
-    attempts = []
-    if launcher and os.path.exists(mpi_bin):
-        attempts.append(([launcher, "-np", str(ranks), mpi_bin] + args, "MPI_Sendrecv (MPICH)"))
-    attempts.append(([shm_bin, "--ranks", str(ranks)] + args, "fork+shared memory"))
-    for cmd, transport in attempts:
-        try:
-            t0 = time.time()
-            p = subprocess.run(cmd, capture_output=True, text=True, timeout=400)
-            line = [l for l in p.stdout.splitlines() if l.startswith("{")]
-            if p.returncode == 0 and line:
-                r = json.loads(line[-1])
-                vendor = None
-                if dtype == "f32" and cmd[0] == launcher:
-                    # the vendor collective the reference reaches with --library mpi
-                    # --pccl-disable-cpp-backend (pccl/reduce_scatter.py:197), same shape
-                    vcmd = [a if a != "ring" else "mpi_block" for a in cmd]
-                    try:
-                        pv = subprocess.run(vcmd, capture_output=True, text=True, timeout=400)
-                        vl = [l for l in pv.stdout.splitlines() if l.startswith("{")]
-                        if pv.returncode == 0 and vl:
-                            vendor = round(json.loads(vl[-1])["GBps"], 3)
-                    except Exception:                         # noqa: BLE001
-                        vendor = None
-                return {"value": round(r["GBps"], 3), "unit": "GB/s", "cores": ranks, "kind": "port",
-                        "mpi_reduce_scatter_block_GBps": vendor,
-                        "ms_per_call": round(r["ms_per_call"], 3), "host_cores": host_cores,
-                        "sample": f"{sample}: ring reduce_scatter of the reference "
-                                  f"(pccl/src/reduce_scatter.cpp:101-155) on host buffers, {ranks} ranks = {ranks} "
-                                  f"processes over {transport}, {dtype}, {block} elements per block "
-                                  f"({ranks * block} per rank), 1 warm-up + {iters} timed calls, "
-                                  f"{time.time() - t0:.1f} s wall"}
-        except Exception:                                     # noqa: BLE001
-            continue
-    return {"value": None, "unit": "GB/s", "cores": 0, "kind": "port", "sample": "baseline program failed"}
+    head, transport, wall = _cpu_leg(ranks, dtype, block, iters, ["ring"], "0.01" if dtype == "bf16" else "1.0")
+    # BASELINE configuration 1, the one the reference can run on CPUs: P = 4, fp32, blocks of 4 Mi elements
+    c1_ranks = min(4, ranks if ranks >= 2 else 1)
+    c1, c1_transport, c1_wall = _cpu_leg(c1_ranks, "f32", 1 << 22, 20, ["ring", "mpi_block"], "1.0")
+    cfg1 = {
+        "ring_GBps": round(c1["ring"]["GBps"], 3) if "ring" in c1 else None,
+        "ring_ms_per_call": round(c1["ring"]["ms_per_call"], 3) if "ring" in c1 else None,
+        "mpi_reduce_scatter_block_GBps": round(c1["mpi_block"]["GBps"], 3) if "mpi_block" in c1 else None,
+        "mpi_reduce_scatter_block_ms_per_call": round(c1["mpi_block"]["ms_per_call"], 3) if "mpi_block" in c1 else None,
+        "cores": c1_ranks,
+        "sample": f"ring reduce_scatter, P = {c1_ranks}, fp32, {c1_ranks << 22} elements per rank: the reference's ring "
+                  f"(pccl/src/reduce_scatter.cpp:101-155) and MPI_Reduce_scatter_block (pccl/reduce_scatter.py:197) on host "
+                  f"buffers, {c1_ranks} processes over {c1_transport}, 1 warm-up + 20 timed calls each, {c1_wall:.1f} s wall",
+    }
+    if "ring" not in head:
+        return {"value": None, "unit": "GB/s", "cores": 0, "kind": "port", "sample": "baseline program failed", "cfg1": cfg1}
+    r = head["ring"]
+    return {"value": round(r["GBps"], 3), "unit": "GB/s", "cores": ranks, "kind": "port",
+            "ms_per_call": round(r["ms_per_call"], 3), "host_cores": host_cores,
+            "sample": f"{sample}: ring reduce_scatter of the reference "
+                      f"(pccl/src/reduce_scatter.cpp:101-155) on host buffers, {ranks} ranks = {ranks} "
+                      f"processes over {transport}, {dtype}, {block} elements per block "
+                      f"({ranks * block} per rank), 1 warm-up + {iters} timed calls, {wall:.1f} s wall",
+            "cfg1": cfg1}
 
 
 # ---------------------------------------------------------------------------

@@ -47,16 +47,16 @@ def test_counter_traffic_is_tied_to_the_kernel_sources(monkeypatch):
     assert table["source_sha256_16"] == bench.source_hash(), \
         "profiles/traffic.json was recorded with other kernel sources: regenerate the counter summaries"
     lib = _Tuning(dict(table["tuning"]))
-    got, why = bench.profiled_traffic("cfg2", "steps", "k_add_segs", lib, 1.0)
-    assert why is None and got == table["entries"]["cfg2:steps:k_add_segs"]
+    got, why = bench.profiled_traffic("cfg2", "steps", "k_add_rows", lib, 1.0)
+    assert why is None and got == table["entries"]["cfg2:steps:k_add_rows"]
     assert abs(got / (3 * 8 * (32 << 20) * 2 / 2) - 1) < 0.01          # ~ the algorithmic bytes of one launch
     # another size, another tuning, an unknown row, other sources: no figure, and the reason
-    assert bench.profiled_traffic("cfg2", "steps", "k_add_segs", lib, 0.5)[0] is None
+    assert bench.profiled_traffic("cfg2", "steps", "k_add_rows", lib, 0.5)[0] is None
     other = _Tuning(dict(table["tuning"], unroll=8))
-    assert bench.profiled_traffic("cfg2", "steps", "k_add_segs", other, 1.0)[0] is None
-    assert "no counter run" in bench.profiled_traffic("cfg9", "steps", "k_add_segs", lib, 1.0)[1]
+    assert bench.profiled_traffic("cfg2", "steps", "k_add_rows", other, 1.0)[0] is None
+    assert "no counter run" in bench.profiled_traffic("cfg9", "steps", "k_add_rows", lib, 1.0)[1]
     monkeypatch.setattr(bench, "source_hash", lambda: "0" * 16)
-    got, why = bench.profiled_traffic("cfg2", "steps", "k_add_segs", lib, 1.0)
+    got, why = bench.profiled_traffic("cfg2", "steps", "k_add_rows", lib, 1.0)
     assert got is None and "other kernel sources" in why
 
 
