@@ -745,6 +745,22 @@ def latency_sweep(steps, warmup, device):
     return rows
 
 
+def latency_from_c():
+    """The same small-message table measured from plain C (csrc/examples/latency_from_c.c, built by
+    `make -C sc2025-pccl-reproducer_amd/csrc example`): what the C ABI itself costs per call."""
+    exe = os.path.join(ROOT, "sc2025-pccl-reproducer_amd", "csrc", "build", "latency_from_c")
+    if not os.path.exists(exe):
+        return {"error": "csrc/build/latency_from_c is not built"}
+    try:
+        p = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+        line = [l for l in p.stdout.splitlines() if l.startswith("[")]
+        if p.returncode == 0 and line:
+            return json.loads(line[-1])
+        return {"error": f"exit code {p.returncode}: {p.stderr[-200:]}"}
+    except Exception as e:                                    # noqa: BLE001
+        return {"error": str(e)}
+
+
 def drop_in(device, steps=5, warmup=2):
     """Wall time of the reference-shaped per-rank calls at the cfg2 size: 8
     virtual ranks (one Python thread each, as `mpirun -np 8` would start them)
@@ -1006,7 +1022,8 @@ def main():
             "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
             "config": {"workload": "latency: bf16 messages of 4 KiB .. 1 MiB; value = accumulate at 1 MiB; "
                                    "microseconds per call include the Python/ctypes launch path",
-                       "latency_us": rows}, "roofline": None, "cpu_baseline": None}), flush=True)
+                       "latency_us": rows, "latency_c_us": latency_from_c()},
+            "roofline": None, "cpu_baseline": None}), flush=True)
         return 0
 
     everything = args.workload == "all"
@@ -1072,6 +1089,7 @@ def main():
                 run_group(name)
         rows.sort(key=lambda r: ALL_ROWS.index((r["workload"], r["mode"])))
         extra["latency_us"] = latency_sweep(50, 10, device)
+        extra["latency_c_us"] = latency_from_c()
         extra["ceilings"] = ceilings(10, 3, device)
         torch.cuda.empty_cache()
         extra["drop_in"] = drop_in(device)

@@ -129,3 +129,20 @@ def test_library_called_from_plain_c():
     assert os.path.exists(exe), "not built: make -C sc2025-pccl-reproducer_amd/csrc example"
     p = subprocess.run([exe], capture_output=True, text=True, timeout=120)
     assert p.returncode == 0 and p.stdout.strip() == "OK", (p.returncode, p.stdout, p.stderr)
+
+
+@pytest.mark.gpu
+def test_latency_program_in_plain_c():
+    """csrc/examples/latency_from_c.c: every entry point it times (also through a
+    captured and replayed HIP graph) runs from C, and a fused 8-rank collective of
+    a small message costs a few microseconds, far below its 7 per-step launches."""
+    import json
+    exe = os.path.join(ROOT, "sc2025-pccl-reproducer_amd", "csrc", "build", "latency_from_c")
+    assert os.path.exists(exe), "not built: make -C sc2025-pccl-reproducer_amd/csrc example"
+    p = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0, (p.returncode, p.stderr)
+    rows = json.loads(p.stdout)
+    assert [r["bytes"] for r in rows] == [4096 << i for i in range(9)]
+    for r in rows:
+        assert 0 < r["ring_rs_p8_fused_us"] < r["ring_rs_p8_steps_us"]
+        assert 0 < r["ring_rs_p8_steps_graph_us"] and 0 < r["accumulate_us"] < 100
