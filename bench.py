@@ -89,7 +89,7 @@ def parse_args():
                          "FETCH_SIZE / WRITE_SIZE readings scale the hardware counters of a rocprofv3 --pmc run")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="launch tuning of the library: any key of pccl_hip_set_tuning (grid_cap, unroll, unroll_copy, "
-                         "nt_load, nt_store, lds_pad*, launch_mib, gather_strip, gather_split, unroll_gather, gather_nt)")
+                         "nt_load, nt_store, add_rows, wg_kway, lds_pad_*, gather_strip, gather_split, unroll_gather, gather_nt)")
     return ap.parse_args()
 
 
@@ -946,8 +946,8 @@ def cpu_baseline(info):
 
 # ---------------------------------------------------------------------------
 
-TUNING_KEYS = ("grid_cap", "unroll", "add_rows", "launch_mib_rows", "wg_kway", "unroll_copy", "nt_load", "nt_store", "launch_mib", "gather_strip",
-               "gather_split", "unroll_gather", "gather_nt", "lds_pad", "lds_pad_copy", "lds_pad_kway",
+TUNING_KEYS = ("grid_cap", "unroll", "add_rows", "wg_kway", "unroll_copy", "nt_load", "nt_store", "gather_strip",
+               "gather_split", "unroll_gather", "gather_nt", "lds_pad_copy", "lds_pad_kway",
                "lds_pad_gather")
 
 

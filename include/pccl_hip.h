@@ -321,16 +321,23 @@ int pccl_hip_probe_mix(const void* const* reads, int nr, void* const* writes,
                        void* stream);
 
 /* ---- launch tuning (for measurement) ------------------------------------
- * key: "grid_cap" (max workgroups per launch, 0 = one tile per workgroup),
- *      "unroll"   (128-bit vectors per thread per operand of the add kernels:
- *                  1, 2, 4 or 8), "unroll_copy" (the same for the copy kernels),
+ * key: "grid_cap" (max workgroups per launch of the 256-thread kernels,
+ *                  0 = one tile per workgroup),
+ *      "add_rows" (1, the default: adds over contiguous 16-byte aligned
+ *                  segments run in the lean one-wave kernels, one 128-bit
+ *                  vector per thread; 0: everything in the general kernels),
+ *      "unroll"   (128-bit vectors per thread per operand of the general add
+ *                  kernels: 1, 2, 4 or 8), "unroll_copy" (the same for the copy
+ *                  kernels),
  *      "nt_load" / "nt_store" (non-temporal global loads / stores: 1 always,
  *                  0 never, -1, the default: for calls whose footprint exceeds
  *                  the Infinity Cache and the L2s, 288 MiB),
- *      "lds_pad" / "lds_pad_copy" / "lds_pad_kway" / "lds_pad_gather" (bytes of
- *                  unused LDS per workgroup, 0..65536: bounds the workgroups
- *                  resident per CU; -1, the default of all but lds_pad,
- *                  lets the launch choose),
+ *      "wg_kway"  (threads per workgroup of the fused reduce: 64, 256, or -1,
+ *                  the default: 64 with loads in pairs for streams from HBM,
+ *                  256 for operands that fit the caches),
+ *      "lds_pad_copy" / "lds_pad_kway" / "lds_pad_gather" (bytes of unused LDS
+ *                  per workgroup, 0..65536: bounds the workgroups resident per
+ *                  CU; -1, the default, lets the launch choose),
  *      "unroll_gather" (vectors per thread of the all_gather placement kernels:
  *                  1, 2, 4, 8; 0, the default: one in the multicast kernel,
  *                  four in the time-blocked one),
@@ -343,11 +350,10 @@ int pccl_hip_probe_mix(const void* const* reads, int nr, void* const* writes,
  *      "gather_split"  (multicast kernel: workgroups sharing one shard tile,
  *                  each storing to 1/gather_split of the outputs;
  *                  0, the default = four outputs per workgroup),
- *      "gather_nt" (non-temporal stores in both kernels: 1, 0 or -1 as above),
- *      "launch_mib" (a step of the add kernels goes out as equal launches that
- *                  move about this many MiB each, a fused reduce over at most
- *                  16 shards as launches 1.5 times as large; 0 = always one
- *                  launch; default 768.  Copies are always one launch).
+ *      "gather_nt" (non-temporal stores in both kernels: 1, 0 or -1 as above).
+ * Every default that is not the plain setting is backed by an A/B measurement
+ * over fresh processes on MI355X; a setting whose gain was inside the
+ * run-to-run spread has been removed.
  * Returns 0, or PCCL_HIP_EINVAL for an unknown key or value.
  * The settings are process-wide: besides the per-thread error message, they,
  * the launch counter below and the per-device address of the built-in scratch

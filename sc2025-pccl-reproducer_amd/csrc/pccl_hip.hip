@@ -74,12 +74,10 @@ std::atomic<long> g_grid_cap{0};
 std::atomic<long> g_unroll{4};        // vectors per thread and operand, general add kernels
 // Aligned contiguous adds go to the lean one-wave kernels (k_add_rows, k_rh_rows); 0 = always the general kernels
 std::atomic<long> g_add_rows{1};
-std::atomic<long> g_launch_mib_rows{0};   // traffic per launch of the lean add kernels, MiB (0 = a step is one launch)
 std::atomic<long> g_unroll_copy{2};   // ... copy kernels (two 4 KiB chunks per workgroup, 8 chunks apart: see copy_vec)
 // Unused dynamic LDS requested per workgroup, only to bound how many workgroups
 // share a CU (160 KiB of LDS): the fewer are resident, the narrower the address
 // window the chip streams from at any moment.  0 = as many as fit (8).
-std::atomic<long> g_lds_pad{0};        // add kernels
 std::atomic<long> g_lds_pad_copy{-1};  // copy kernels; -1 = chosen per launch (see copy_lds_pad)
 std::atomic<long> g_lds_pad_kway{-1};  // fused reduce; -1 = chosen per launch (see launch_kway)
 std::atomic<long> g_wg_kway{-1};       // threads per workgroup of the fused reduce: 64, 256, or -1 = 64 for streams from HBM
@@ -90,7 +88,6 @@ std::atomic<long> g_unroll_gather{0};  // vectors per thread in the all_gather p
 std::atomic<long> g_gather_strip{-1};  // work items per XCD and strip of the time-blocked gather; 0 = the multicast kernel, -1 = chosen per launch
 std::atomic<long> g_gather_strip_from{-1};  // shortest longest-shard (bytes) the time-blocked gather is chosen for when gather_strip = -1
 std::atomic<unsigned long long> g_launches{0};   // kernel launches issued so far
-std::atomic<long> g_launch_mib{768};   // traffic per launch of the add kernels, MiB (0 = a step is one launch whatever its size)
 // Non-temporal loads / stores: 1 = always, 0 = never, -1 = by the footprint of
 // the call.  Data that fits the 256 MB Infinity Cache and the L2s is better left
 // cacheable (the next step or call finds it there: a P=8 ring reduce_scatter of
@@ -147,34 +144,16 @@ unsigned grid_for(size_t total_tiles) {
   return (unsigned)g;
 }
 
-// Calls launch(span, grid) for consecutive, equal spans of the `items` work
-// items of a schedule step, each moving about target_mib MiB (item_bytes per
-// work item; 0 = one span); span bounds are multiples of `multiple`.
-// On MI355X the add kernels slow down over the length of a launch: 12 GiB of
-// traffic in one launch runs at 6.0 TB/s, as launches of 0.75-1.5 GiB at 6.4;
-// pieces under 0.5 GiB lose again to the drain at the end of every launch.
-// Copies and the multicast gather do not show it; the fused reduce gains 2 %
-// for 8 and 16 shards and loses for 32 (its workgroups live k loads long, and
-// so does the drain), see KwayLaunch.
+// One launch over the `items` work items of a schedule step: launch(span, grid).
+// (Steps of the 256-thread add kernels used to go out as several launches of
+// bounded size; with the one-wave kernels serving the aligned case that measured
+// inside the run-to-run spread on MI355X and was dropped.)
 template <class F>
-void for_spans(size_t items, size_t item_bytes, size_t multiple, long target_mib, F&& launch) {
+void for_spans(size_t items, F&& launch) {
   if (items == 0) return;
-  size_t per = items;
-  if (target_mib > 0 && item_bytes > 0) {
-    const double total = (double)items * (double)item_bytes;
-    size_t pieces = (size_t)(total / ((double)target_mib * 1048576.0) + 0.5);
-    if (pieces < 1) pieces = 1;
-    per = (items + pieces - 1) / pieces;
-    per = (per + multiple - 1) / multiple * multiple;
-  }
-  for (size_t w0 = 0; w0 < items; w0 += per) {
-    const size_t w1 = items - w0 < per ? items : w0 + per;
-    launch(Span{(uint32_t)w0, (uint32_t)w1}, grid_for(w1 - w0));
-    g_launches.fetch_add(1, std::memory_order_relaxed);
-  }
+  launch(Span{0u, (uint32_t)items}, grid_for(items));
+  g_launches.fetch_add(1, std::memory_order_relaxed);
 }
-
-long add_launch_mib() { return g_launch_mib.load(std::memory_order_relaxed); }
 
 size_t tiles_for(size_t nbytes, int unroll, int threads = kThreads) {
   // one extra vector covers the shift of the body behind an unaligned head
@@ -251,8 +230,8 @@ struct AddLaunch {
   hipStream_t stream;
   template <int U, bool NTL, bool NTS, int T>
   void run() const {
-    const unsigned lds = (unsigned)g_lds_pad.load();
-    for_spans((size_t)count * pc.s1 * pc.s2 * tiles, (size_t)3 * T * 16 * U, 1, add_launch_mib(), [&](Span span, unsigned grid) {
+    const unsigned lds = 0;
+    for_spans((size_t)count * pc.s1 * pc.s2 * tiles, [&](Span span, unsigned grid) {
       if (dtype == PCCL_HIP_F32)
         PCCL_LAUNCH((k_add_segs<OpF32, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *segs, count, pc, tiles, aligned, span);
       else
@@ -265,46 +244,14 @@ struct AddLaunch {
   }
 };
 
-// Calls launch(row0, nrows, tile0, ntiles) for the launches of a lean add step:
-// `rows` segments of `tiles` one-vector-per-thread tiles each, in pieces of
-// about target_mib MiB (0 = one launch) cut between rows where a piece holds
-// whole rows, inside a row otherwise.
-template <class F>
-void for_rows(int rows, size_t tiles, size_t tile_bytes, long target_mib, F&& launch) {
-  if (rows <= 0 || tiles == 0) return;
-  int rows_per = rows;
-  size_t tiles_per = tiles;
-  if (target_mib > 0) {
-    const double total = (double)rows * (double)tiles * (double)tile_bytes;
-    size_t pieces = (size_t)(total / ((double)target_mib * 1048576.0) + 0.5);
-    if (pieces < 1) pieces = 1;
-    if (pieces <= (size_t)rows) {
-      rows_per = (int)(((size_t)rows + pieces - 1) / pieces);
-    } else {
-      rows_per = 1;
-      const size_t per_row = (pieces + (size_t)rows - 1) / (size_t)rows;
-      tiles_per = (tiles + per_row - 1) / per_row;
-    }
-  }
-  if (rows_per > 65535) rows_per = 65535;
-  if (tiles_per > kMaxGrid) tiles_per = kMaxGrid;
-  for (int r0 = 0; r0 < rows; r0 += rows_per) {
-    const int nr = rows - r0 < rows_per ? rows - r0 : rows_per;
-    for (size_t t0 = 0; t0 < tiles; t0 += tiles_per) {
-      const size_t nt = tiles - t0 < tiles_per ? tiles - t0 : tiles_per;
-      launch(r0, nr, (uint32_t)t0, (unsigned)nt);
-      g_launches.fetch_add(1, std::memory_order_relaxed);
-    }
-  }
-}
-
 // The lean add for `count` contiguous, aligned segments of n elements.
 void launch_add_rows(const AddSegs& segs, int count, size_t n, int dtype, const Tune& t, hipStream_t stream) {
   const size_t nvec = n * esize_of(dtype) / 16;
   const size_t tiles = (nvec + kRowThreads - 1) / kRowThreads;
-  for_rows(count, tiles, (size_t)3 * kRowThreads * 16, g_launch_mib_rows.load(std::memory_order_relaxed),
-           [&](int row0, int nrows, uint32_t tile0, unsigned ntiles) {
-#define PCCL_ROWS(OP, L, S) PCCL_LAUNCH((k_add_rows<OP, L, S>), dim3(ntiles, (unsigned)nrows), dim3(kRowThreads), 0, stream, segs, row0, nvec, tile0)
+  {
+    const int row0 = 0;
+    const uint32_t tile0 = 0;
+#define PCCL_ROWS(OP, L, S) PCCL_LAUNCH((k_add_rows<OP, L, S>), dim3((unsigned)tiles, (unsigned)count), dim3(kRowThreads), 0, stream, segs, row0, nvec, tile0)
     if (dtype == PCCL_HIP_F32) {
       if (t.ntl) { if (t.nts) PCCL_ROWS(OpF32, true, true); else PCCL_ROWS(OpF32, true, false); }
       else { if (t.nts) PCCL_ROWS(OpF32, false, true); else PCCL_ROWS(OpF32, false, false); }
@@ -313,7 +260,8 @@ void launch_add_rows(const AddSegs& segs, int count, size_t n, int dtype, const 
       else { if (t.nts) PCCL_ROWS(OpBF16, false, true); else PCCL_ROWS(OpBF16, false, false); }
     }
 #undef PCCL_ROWS
-  });
+    g_launches.fetch_add(1, std::memory_order_relaxed);
+  }
 }
 
 // True if every piece of every operand starts on a 16-byte boundary and is a
@@ -332,7 +280,7 @@ int launch_add_pieces(const AddSegs& segs, int count, const Pieces& pc, int dtyp
   bool aligned = pieces_aligned(pc, esize_of(dtype));
   for (int s = 0; s < count && aligned; ++s) aligned = is16(segs.dst[s]) && is16(segs.a[s]) && is16(segs.b[s]);
   if (aligned && pc.s1 == 1 && pc.s2 == 1 && g_add_rows.load(std::memory_order_relaxed) &&
-      pc.len * esize_of(dtype) / 16 <= kMaxWorkItems * (size_t)kRowThreads) {
+      pc.len * esize_of(dtype) / 16 <= (size_t)kMaxGrid * kRowThreads) {
     launch_add_rows(segs, count, pc.len, dtype, t, stream);
     return launch_status(what);
   }
@@ -367,7 +315,7 @@ struct CopyLaunch {
   template <int U, bool NTL, bool NTS>
   void operator()() const {
     const unsigned lds = copy_lds_pad(traffic);
-    for_spans((size_t)count * tiles, 2 * kTileBytes * U, 1, 0, [&](Span span, unsigned grid) {
+    for_spans((size_t)count * tiles, [&](Span span, unsigned grid) {
       PCCL_LAUNCH((k_copy_segs<U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *segs, count, tiles, aligned, span);
     });
   }
@@ -400,7 +348,7 @@ struct CopyPiecesLaunch {
   template <int U, bool NTL, bool NTS>
   void operator()() const {
     const unsigned lds = copy_lds_pad(2 * (size_t)count * pc.s1 * pc.s2 * pc.len);
-    for_spans((size_t)count * pc.s1 * pc.s2 * tiles, 2 * kTileBytes * U, 1, 0, [&](Span span, unsigned grid) {
+    for_spans((size_t)count * pc.s1 * pc.s2 * tiles, [&](Span span, unsigned grid) {
       PCCL_LAUNCH((k_copy_pieces<U, NTL, NTS>), dim3(grid), dim3(kThreads), lds, stream, *segs, count, pc, tiles, aligned, span);
     });
   }
@@ -428,8 +376,8 @@ struct RhLaunch {
   hipStream_t stream;
   template <int U, bool NTL, bool NTS, int T>
   void run() const {
-    const unsigned lds = (unsigned)g_lds_pad.load();
-    for_spans((size_t)P * tiles, (size_t)3 * T * 16 * U, 1, add_launch_mib(), [&](Span span, unsigned grid) {
+    const unsigned lds = 0;
+    for_spans((size_t)P * tiles, [&](Span span, unsigned grid) {
       if (dtype == PCCL_HIP_F32)
         PCCL_LAUNCH((k_rh_round<OpF32, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *args, P, B, round, from_src, to_outs, tiles, aligned, span);
       else
@@ -452,9 +400,7 @@ struct GatherLaunch {
   // Plain loads whatever the tuning says; the stores follow their own setting.
   template <int U, bool NTL, bool NTS>
   void operator()() const {
-    // a work item reads a tile and stores it to its share of the outputs
-    const size_t item_bytes = kTileBytes * U * (1 + ((size_t)nout + split - 1) / split);
-    for_spans((size_t)P * tiles * (size_t)split, item_bytes, (size_t)split, 0, [&](Span span, unsigned grid) {
+    for_spans((size_t)P * tiles * (size_t)split, [&](Span span, unsigned grid) {
       if (nt)
         PCCL_LAUNCH((k_gather_multicast<U, false, true>), dim3(grid), dim3(kThreads), lds_pad, stream, *args, P, nout, tiles, split, span);
       else
@@ -471,7 +417,7 @@ struct TransposeLaunch {
   hipStream_t stream;
   template <int U, bool NTL, bool NTS>
   void operator()() const {
-    for_spans(rows * cols * tiles, 2 * kTileBytes * U, 1, 0, [&](Span span, unsigned grid) {
+    for_spans(rows * cols * tiles, [&](Span span, unsigned grid) {
       PCCL_LAUNCH((k_block_transpose<U, NTL, NTS>), dim3(grid), dim3(kThreads), 0, stream, dst, src, rows, cols, m, tiles, aligned, span);
     });
   }
@@ -489,11 +435,11 @@ struct KwayLaunch {
   hipStream_t stream;
 
   template <class Acc, int U, bool NTL, bool NTS, int T, int PF>
-  void run_wg(long span_mib) const {
+  void run_wg() const {
     static_assert(U == 1, "the fused reduce is launched with one vector per thread");
 #define PCCL_KWAY(KV) \
   PCCL_LAUNCH((k_reduce_kway<Acc, KV, U, NTL, NTS, T, PF>), dim3(grid), dim3(T), lds_pad, stream, *args, k, g, nout, n, first0, tiles, span)
-    for_spans((size_t)nout * tiles, (size_t)T * 16 * U * ((size_t)k + 1), 1, span_mib, [&](Span span, unsigned grid) {
+    for_spans((size_t)nout * tiles, [&](Span span, unsigned grid) {
       if (order == PCCL_HIP_ORDER_RING) { PCCL_KWAY(0); return; }
       switch (k) {
         case 2: PCCL_KWAY(2); break;
@@ -511,13 +457,9 @@ struct KwayLaunch {
   void run() const {
     if constexpr (NTL && NTS) {
       // streams from HBM: one-wave workgroups, ring-order loads in pairs whatever k, one launch
-      if (threads == kRowThreads) { run_wg<Acc, U, NTL, NTS, kRowThreads, 2>(0); return; }
+      if (threads == kRowThreads) { run_wg<Acc, U, NTL, NTS, kRowThreads, 2>(); return; }
     }
-    // 256 threads: folds over at most 16 shards go out as launches 1.5 times (butterfly order, +2-4 %) or
-    // 3 times (ring order, +1-2 %) the size of the add kernels'; longer folds lose more to the drain of a
-    // launch than they gain, and stay one launch
-    const long span_mib = k > 16 ? 0 : order == PCCL_HIP_ORDER_RING ? add_launch_mib() * 3 : add_launch_mib() * 3 / 2;
-    run_wg<Acc, U, NTL, NTS, kThreads, kFoldPairedFrom>(span_mib);
+    run_wg<Acc, U, NTL, NTS, kThreads, kFoldPairedFrom>();
   }
 
   template <int U, bool NTL, bool NTS>
@@ -529,46 +471,23 @@ struct KwayLaunch {
   }
 };
 
-// Unused LDS per workgroup of the fused reduce, chosen for a launch.  It takes
-// the room of further workgroups on a CU (160 KiB of LDS: 21 KiB leave 7
-// resident, 24 KiB 6, 30 KiB 5, 32 KiB 4, 48 KiB 3; 8 without), and fewer
-// resident workgroups narrow the window each of the k streams has in flight.
-// Measured on MI355X on 4 GiB of operands, against 8 per CU, operands carved
-// from one allocation and allocated one by one alike:
-//   ring order, bf16:   3-15 shards 7 per CU +2-5 % (6 is as good or better for
-//                       8 and more shards in some placements of the operands'
-//                       pages and 2 % worse in others), 16 and more 4 +5-8 %;
-//   ring order, fp32:   5-15 shards 6 +1-4 %, 16-23 shards 4 +6-8 %, 24 and more
-//                       3 +7-14 % (4 below 768 MiB of traffic);
-//   two-level ring:     bf16 7 (up to 8 shards) or 6, +2-4 %; fp32 5, +4-8 %;
-//   halving butterfly:  fp32 8 and 16 shards 4 per CU, +2-7 %; its other sizes
-//                       and bf16 gain in one placement what they lose in another.
-// All of it holds for streams from HBM only: operands that fit the caches (up
-// to about 256 MiB of traffic) lose 2-9 % with fewer workgroups, so the
-// footprint rule of the non-temporal hints decides here too.
+// Unused LDS per workgroup of the fused reduce, chosen for a launch: it takes the
+// room of further workgroups on a CU (160 KiB of LDS), and fewer resident waves
+// narrow the window each of the k streams has in flight.  Only the one-wave
+// workgroups that streams from HBM get are limited; operands that fit the caches
+// (the footprint rule of the non-temporal hints) and 256-thread workgroups run
+// at full occupancy.  8 KiB leave 20 waves on a CU, 11 KiB 14, 16 KiB 10; 32
+// without.  Measured on MI355X (fraction of 8 TB/s at 32 / 20 / 16 / 14 waves per
+// CU): ring order, 8 bf16 shards 0.79 / 0.835 / 0.80 / 0.745, 16 bf16 shards
+// 0.77 / 0.81 / 0.81 / 0.765, 64 bf16 shards 0.76 / 0.79 / 0.79 / 0.77, 32 fp32
+// shards 0.76 / 0.81 / 0.82 / 0.84; halving order, 8 bf16 and 16 fp32 shards
+// 0.76 / 0.785 / 0.79 / 0.80, 64 bf16 shards of 1 GiB 0.79 / 0.81 / - / 0.855.
+// Launches below 512 MiB of traffic are too short to profit.
 long kway_lds_pad(int k, int g, int dtype, int order, size_t traffic, int threads) {
-  if (!stream_hint(-1, traffic)) return 0;
-  const bool f32 = dtype == PCCL_HIP_F32;
-  if (threads == kRowThreads) {
-    // One-wave workgroups: 8 KiB leave 20 waves on a CU, 11 KiB 14, 16 KiB 10; 32 without.  Measured on
-    // MI355X (fraction of 8 TB/s at 32 / 20 / 16 / 14 waves per CU): ring order, 8 bf16 shards
-    // 0.79 / 0.835 / 0.80 / 0.745, 16 bf16 shards 0.77 / 0.81 / 0.81 / 0.765, 64 bf16 shards
-    // 0.76 / 0.79 / 0.79 / 0.77, 32 fp32 shards 0.76 / 0.81 / 0.82 / 0.84; halving order, 8 bf16 and
-    // 16 fp32 shards 0.76 / 0.785 / 0.79 / 0.80, 64 bf16 shards of 1 GiB 0.79 / 0.81 / - / 0.855 (and
-    // 0.855 at 10, 0.80 at 8).  Launches below 512 MiB of traffic are too short to profit.
-    if (traffic < ((size_t)512 << 20)) return 0;
-    if (order == PCCL_HIP_ORDER_RING) return f32 && k >= 24 ? 11264 : 8192;
-    return 11264;
-  }
-  if (order == PCCL_HIP_ORDER_RING) {
-    if (g >= k) {
-      if (f32) return k >= 24 ? (traffic >= ((size_t)768 << 20) ? 49152 : 32768) : k >= 16 ? 32768 : k >= 5 ? 24576 : 0;
-      return k >= 16 ? 32768 : k >= 3 ? 21504 : 0;
-    }
-    if (f32) return 30720;
-    return k <= 8 ? 21504 : 24576;
-  }
-  return f32 && (k == 8 || k == 16) ? 32768 : 0;
+  (void)g;
+  if (threads != kRowThreads || !stream_hint(-1, traffic) || traffic < ((size_t)512 << 20)) return 0;
+  if (order == PCCL_HIP_ORDER_RING) return dtype == PCCL_HIP_F32 && k >= 24 ? 11264 : 8192;
+  return 11264;
 }
 
 // g = size of the inner groups of a two-level ring order (g >= k: one level).
@@ -763,18 +682,14 @@ int pccl_hip_set_tuning(const char* key, long value) {
     g_wg_kway = value;
   } else if (!strcmp(key, "add_rows")) {
     g_add_rows = value != 0;
-  } else if (!strcmp(key, "launch_mib_rows")) {
-    if (value < 0) return fail(PCCL_HIP_EINVAL, "set_tuning: launch_mib_rows must be >= 0");
-    g_launch_mib_rows = value;
   } else if (!strcmp(key, "unroll_copy")) {
     if (value != 1 && value != 2 && value != 4 && value != 8)
       return fail(PCCL_HIP_EINVAL, "set_tuning: unroll_copy must be 1, 2, 4 or 8");
     g_unroll_copy = value;
-  } else if (!strcmp(key, "lds_pad") || !strcmp(key, "lds_pad_copy") || !strcmp(key, "lds_pad_kway")) {
-    const long lowest = !strcmp(key, "lds_pad") ? 0 : -1;   // -1: the copies and the fused reduce pick per launch
-    if (value < lowest || value > 65536)
-      return fail(PCCL_HIP_EINVAL, "set_tuning: %s must be in [%ld, 65536]", key, lowest);
-    (!strcmp(key, "lds_pad") ? g_lds_pad : !strcmp(key, "lds_pad_copy") ? g_lds_pad_copy : g_lds_pad_kway) = value;
+  } else if (!strcmp(key, "lds_pad_copy") || !strcmp(key, "lds_pad_kway")) {
+    if (value < -1 || value > 65536)   // -1: the copies and the fused reduce pick per launch
+      return fail(PCCL_HIP_EINVAL, "set_tuning: %s must be in [-1, 65536]", key);
+    (!strcmp(key, "lds_pad_copy") ? g_lds_pad_copy : g_lds_pad_kway) = value;
   } else if (!strcmp(key, "lds_pad_gather")) {
     if (value < -1 || value > 65536) return fail(PCCL_HIP_EINVAL, "set_tuning: lds_pad_gather must be in [-1, 65536]");
     g_lds_pad_gather = value;
@@ -790,9 +705,6 @@ int pccl_hip_set_tuning(const char* key, long value) {
     if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8)
       return fail(PCCL_HIP_EINVAL, "set_tuning: unroll_gather must be 0, 1, 2, 4 or 8");
     g_unroll_gather = value;
-  } else if (!strcmp(key, "launch_mib")) {
-    if (value < 0) return fail(PCCL_HIP_EINVAL, "set_tuning: launch_mib must be >= 0");
-    g_launch_mib = value;
   } else if (!strcmp(key, "gather_nt") || !strcmp(key, "nt_load") || !strcmp(key, "nt_store")) {
     // -1: non-temporal for calls whose footprint exceeds the caches, 0: never, other: always
     const long v = value < 0 ? -1 : value != 0;
@@ -811,9 +723,7 @@ long pccl_hip_get_tuning(const char* key) {
   if (!strcmp(key, "unroll")) return g_unroll;
   if (!strcmp(key, "wg_kway")) return g_wg_kway;
   if (!strcmp(key, "add_rows")) return g_add_rows;
-  if (!strcmp(key, "launch_mib_rows")) return g_launch_mib_rows;
   if (!strcmp(key, "unroll_copy")) return g_unroll_copy;
-  if (!strcmp(key, "lds_pad")) return g_lds_pad;
   if (!strcmp(key, "lds_pad_copy")) return g_lds_pad_copy;
   if (!strcmp(key, "lds_pad_kway")) return g_lds_pad_kway;
   if (!strcmp(key, "lds_pad_gather")) return g_lds_pad_gather;
@@ -822,7 +732,6 @@ long pccl_hip_get_tuning(const char* key) {
   if (!strcmp(key, "gather_strip")) return g_gather_strip;
   if (!strcmp(key, "gather_strip_from")) return g_gather_strip_from;
   if (!strcmp(key, "gather_nt")) return g_gather_nt;
-  if (!strcmp(key, "launch_mib")) return g_launch_mib;
   if (!strcmp(key, "nt_load")) return g_nt_load;
   if (!strcmp(key, "nt_store")) return g_nt_store;
   return -1;
@@ -897,16 +806,17 @@ int pccl_hip_rh_round(void* const* bufs, const void* const* src, void* const* ou
   bool aligned = (B * esize_of(dtype)) % 16 == 0;
   for (int r = 0; r < P && aligned; ++r)
     aligned = is16(args.bufs[r]) && is16(args.src[r]) && is16(args.outs[r]);
-  if (aligned && g_add_rows.load(std::memory_order_relaxed) && count * esize_of(dtype) / 16 <= kMaxWorkItems * (size_t)kRowThreads) {
+  if (aligned && g_add_rows.load(std::memory_order_relaxed) && count * esize_of(dtype) / 16 <= (size_t)kMaxGrid * kRowThreads) {
     const size_t nvec = count * esize_of(dtype) / 16;
     const size_t tiles = (nvec + kRowThreads - 1) / kRowThreads;
     int log2_group = 0;
     while ((1 << log2_group) < (P >> round)) ++log2_group;
     const int from_src = src ? 1 : 0, outs_i = to_outs ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;
-    for_rows(P, tiles, (size_t)3 * kRowThreads * 16, g_launch_mib_rows.load(std::memory_order_relaxed),
-             [&](int row0, int nrows, uint32_t tile0, unsigned ntiles) {
-#define PCCL_RH(OP, L, S) PCCL_LAUNCH((k_rh_rows<OP, L, S>), dim3(ntiles, (unsigned)nrows), dim3(kRowThreads), 0, st, args, row0, log2_group, B, from_src, outs_i, nvec, tile0)
+    {
+      const int row0 = 0;
+      const uint32_t tile0 = 0;
+#define PCCL_RH(OP, L, S) PCCL_LAUNCH((k_rh_rows<OP, L, S>), dim3((unsigned)tiles, (unsigned)P), dim3(kRowThreads), 0, st, args, row0, log2_group, B, from_src, outs_i, nvec, tile0)
       if (dtype == PCCL_HIP_F32) {
         if (t.ntl) { if (t.nts) PCCL_RH(OpF32, true, true); else PCCL_RH(OpF32, true, false); }
         else { if (t.nts) PCCL_RH(OpF32, false, true); else PCCL_RH(OpF32, false, false); }
@@ -915,7 +825,8 @@ int pccl_hip_rh_round(void* const* bufs, const void* const* src, void* const* ou
         else { if (t.nts) PCCL_RH(OpBF16, false, true); else PCCL_RH(OpBF16, false, false); }
       }
 #undef PCCL_RH
-    });
+      g_launches.fetch_add(1, std::memory_order_relaxed);
+    }
     return launch_status(what);
   }
   RhLaunch l{&args, P, round, dtype, src ? 1 : 0, to_outs ? 1 : 0, B,
@@ -1065,7 +976,7 @@ int gather_place_all(void* const* outputs, int nout, const void* const* inputs, 
     if (nts) PCCL_LAUNCH((k_gather_strips<UV, false, true>), dim3(grid), dim3(kThreads), lds, st, args, P, nout, (uint32_t)n_local, (uint32_t)strip, span); \
     else PCCL_LAUNCH((k_gather_strips<UV, false, false>), dim3(grid), dim3(kThreads), lds, st, args, P, nout, (uint32_t)n_local, (uint32_t)strip, span);    \
     break;
-    for_spans((size_t)P * (size_t)nout * kXcds * n_local, 0, 1, 0, [&](Span span, unsigned grid) {
+    for_spans((size_t)P * (size_t)nout * kXcds * n_local, [&](Span span, unsigned grid) {
       switch (U) {
         PCCL_STRIPS(1)
         PCCL_STRIPS(2)

@@ -330,16 +330,17 @@ def test_every_launch_tuning_gives_the_same_bits(target, unroll, nt, grid_cap):
             lib.set_tuning(k, v)
 
 
-@pytest.mark.parametrize("launch_mib", [0, 1, 3])
-def test_bounded_launches_give_the_same_bits(target, launch_mib):
-    """A step that goes out as several launches of bounded size (launch_mib)
-    computes what the single launch computes."""
+@pytest.mark.parametrize("grid_cap", [0, 7])
+def test_ragged_collectives_and_capped_grids(target, grid_cap):
+    """Ragged blocks (the general kernels) through every collective, with one
+    workgroup per tile and with a grid capped to a few workgroups that stride
+    over the tiles."""
     import torch
     from pccl import kernels
     lib = target.native
-    saved = lib.get_tuning("launch_mib")
+    saved = lib.get_tuning("grid_cap")
     try:
-        lib.set_tuning("launch_mib", launch_mib)
+        lib.set_tuning("grid_cap", grid_cap)
         P, B = 4, 150_001
         for dtype in DTYPES:
             ins = make_inputs(P, P * B, dtype, seed=23)
@@ -376,7 +377,7 @@ def test_bounded_launches_give_the_same_bits(target, launch_mib):
         want_t = src.view(torch.int32).view(3, 5, 100_003).transpose(0, 1).reshape(-1)
         assert torch.equal(dst.view(torch.int32), want_t)
     finally:
-        lib.set_tuning("launch_mib", saved)
+        lib.set_tuning("grid_cap", saved)
 
 
 @pytest.mark.parametrize("unroll", [1, 2, 4, 8])
@@ -531,18 +532,16 @@ def test_one_wave_fold_gives_the_same_bits(target, dtype, order):
             lib.set_tuning(k, v)
 
 
-@pytest.mark.parametrize("add_rows,launch_mib_rows", [(0, 0), (1, 1), (1, 3)])
-def test_lean_and_general_add_kernels_agree(target, add_rows, launch_mib_rows):
+@pytest.mark.parametrize("add_rows", [0, 1])
+def test_lean_and_general_add_kernels_agree(target, add_rows):
     """Aligned contiguous adds go to the lean one-wave kernels, everything else
-    (and everything when add_rows = 0) to the general ones; a lean step cut into
-    several launches between rows (3 MiB) or inside rows (1 MiB) computes the same."""
+    (and everything when add_rows = 0) to the general ones."""
     import torch
     from pccl import kernels
     lib = target.native
-    saved = {k: lib.get_tuning(k) for k in ("add_rows", "launch_mib_rows")}
+    saved = {k: lib.get_tuning(k) for k in ("add_rows",)}
     try:
         lib.set_tuning("add_rows", add_rows)
-        lib.set_tuning("launch_mib_rows", launch_mib_rows)
         P, B = 4, 150_000          # blocks of whole vectors: the aligned path
         for dtype in DTYPES:
             ins = make_inputs(P, P * B, dtype, seed=29)
