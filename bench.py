@@ -600,8 +600,10 @@ def ceilings(steps, warmup, device):
     }
     del a, b, c, fa, fb, fc
     # read:write mixes, the best of the probe's shapes (all streams per workgroup or
-    # one stream per workgroup; 1, 2 or 4 vectors per thread), beside the library
-    # kernel of the same mix on the same buffers
+    # one stream per workgroup; 256 threads or one wave per workgroup; 1, 2 or 4 vectors
+    # per thread), beside the library kernel of the same mix on the same buffers.  The
+    # probes are reference points, not bounds: a ratio above 1 says that the library
+    # kernel orders its work better than any of the probe's plain shapes.
     mixes = {}
     for nr, nw, mib in ((2, 1, 1024), (8, 1, 256), (32, 1, 128), (1, 16, 128)):
         nb = mib * MiB
@@ -609,7 +611,7 @@ def ceilings(steps, warmup, device):
         wr = [torch.empty(nb // 4, device=device) for _ in range(nw)]
         rp, wp = [t.data_ptr() for t in rd], [t.data_ptr() for t in wr]
         best, shape = 0.0, None
-        for sh in (0, 1):
+        for sh in (0, 1, 2, 3):
             for u in (1, 2, 4):
                 v = gbps(lambda: lib.probe_mix(rp, wp, nb, sh, u, st), (nr + nw) * nb)
                 if v > best:

@@ -299,12 +299,13 @@ int pccl_hip_all_gather_2d_virtual(void* const* outputs,
                                    const char* algorithm, int mode, void* stream);
 
 /* ---- bandwidth probe (for measurement) --------------------------------------
- * One pure streaming pass over buf[0:nbytes] with the access shape of the
- * kernels above: kind 0 reads every byte (nothing is written), kind 1
- * overwrites every byte with the bf16 pattern of 1.0.  Timing it gives the
- * read and write bandwidth this device actually sustains, the practical
- * ceiling the 2-reads-1-write kernels are judged against.  No counterpart in
- * the reference.  buf must be 16-byte aligned, nbytes >= 4096. */
+ * One pure streaming pass over buf[0:nbytes]: kind 0 reads every byte (nothing
+ * is written; workgroups of 1024 threads, the fastest shape measured for
+ * reads), kind 1 overwrites every byte with the bf16 pattern of 1.0
+ * (workgroups of 256 threads, the fastest for writes).  Timing it gives the
+ * read and write bandwidth this device sustains, reference points beside the
+ * 2-reads-1-write kernels.  No counterpart in the reference.  buf must be
+ * 16-byte aligned, nbytes >= 16384. */
 int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream);
 
 /* A read:write MIX in one launch: nr read streams and nw write streams of
@@ -313,8 +314,13 @@ int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream);
  * what the device sustains for the 2:1 mix of the add kernels, the k:1 mix of
  * the fused reduce or the 1:P mix of the all_gather placement when nothing but
  * the memory system is in the way.  shape 0: workgroup t serves tile t of every
- * stream; shape 1: every workgroup serves one stream.  vectors = 128-bit
- * vectors per thread and stream (1, 2 or 4).  No counterpart in the reference.
+ * stream; shape 1: every workgroup serves one stream; shapes 2 and 3: the same
+ * two with one-wave workgroups (64 threads, the shape of the lean add kernels
+ * and of the fused reduce on streams from HBM).  vectors = 128-bit vectors per
+ * thread and stream (1, 2 or 4).  The best of these shapes is a reference
+ * point, not an upper bound: a library kernel that orders its work in time
+ * (the time-blocked all_gather) runs ahead of all of them.  No counterpart in
+ * the reference.
  * Streams must be 16-byte aligned, nbytes a multiple of 16, nr, nw <= 64. */
 int pccl_hip_probe_mix(const void* const* reads, int nr, void* const* writes,
                        int nw, size_t nbytes, int shape, int vectors,

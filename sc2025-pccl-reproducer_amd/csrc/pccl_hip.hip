@@ -494,6 +494,11 @@ long kway_lds_pad(int k, int g, int dtype, int order, size_t traffic, int thread
 int launch_kway(const KwayArgs& args, int k, int g, int nout, size_t n, int dtype, int order,
                 int first0, int per_hop, hipStream_t stream, const char* what) {
   if (n == 0 || nout == 0) return PCCL_HIP_OK;
+  // an output at an address that is no multiple of its element size would leave the whole fold to the
+  // element-wise path of one workgroup: refused instead
+  for (int j = 0; j < nout; ++j)
+    if ((uintptr_t)args.out[j] % esize_of(dtype))
+      return fail(PCCL_HIP_EINVAL, "%s: output %d is not aligned to its element size (%zu bytes)", what, j, esize_of(dtype));
   const size_t traffic = ((size_t)k + 1) * n * esize_of(dtype) * (size_t)nout;
   const Tune tune = current_tune(false, traffic);
   long wg = g_wg_kway.load(std::memory_order_relaxed);
@@ -1704,22 +1709,22 @@ int pccl_hip_all_gather_2d_virtual(void* const* outputs, const void* const* inpu
 int pccl_hip_probe_stream(int kind, void* buf, size_t nbytes, void* stream) {
   const char* what = "pccl_hip_probe_stream";
   if (kind != 0 && kind != 1) return fail(PCCL_HIP_EINVAL, "%s: kind must be 0 (read) or 1 (write)", what);
-  if (nbytes < 4096) return fail(PCCL_HIP_EINVAL, "%s: buffer must hold at least 4096 bytes", what);
+  if (nbytes < 16384) return fail(PCCL_HIP_EINVAL, "%s: buffer must hold at least 16384 bytes", what);
   if (!buf || ((uintptr_t)buf & 15u)) return fail(PCCL_HIP_EINVAL, "%s: buffer must be 16-byte aligned", what);
   const size_t nvec = nbytes / 16;
-  // vectors per thread: four for the read stream, one for the write stream, the
-  // shapes that sustain the most on MI355X (writes: 6.8 TB/s with 4 KiB per
-  // workgroup against 6.0 with 16 KiB)
-  const size_t per_tile = (size_t)kThreads * (kind == 0 ? 4 : 1);
+  // the shapes that sustain the most on MI355X: reads, workgroups of 1024 threads with one vector each
+  // (7.5 TB/s over 2 GiB against 7.0 with 256 threads); writes, 256 threads with one vector each
+  // (6.8 TB/s with 4 KiB per workgroup against 6.2 with 16 KiB)
+  const size_t per_tile = kind == 0 ? 1024 : (size_t)kThreads;
   const size_t tiles = (nvec + per_tile - 1) / per_tile;
   if (tiles > kMaxGrid) return fail(PCCL_HIP_EINVAL, "%s: buffer too large", what);
   hipStream_t st = (hipStream_t)stream;
   if (kind == 0)
-    PCCL_LAUNCH((k_probe_read<4, true>), dim3((unsigned)tiles), dim3(kThreads), 0, st,
-                       (const u32x4*)buf, (u32x4*)buf, nvec);
+    PCCL_LAUNCH((k_probe_read<1, true, 1024>), dim3((unsigned)tiles), dim3(1024), 0, st,
+                (const u32x4*)buf, (u32x4*)buf, nvec);
   else
-    PCCL_LAUNCH((k_probe_write<1, false>), dim3((unsigned)tiles), dim3(kThreads), 0, st, (u32x4*)buf, nvec,
-                       0x3f803f80u);
+    PCCL_LAUNCH((k_probe_write<1, false, kThreads>), dim3((unsigned)tiles), dim3(kThreads), 0, st, (u32x4*)buf, nvec,
+                0x3f803f80u);
   g_launches.fetch_add(1, std::memory_order_relaxed);
   return launch_status(what);
 }
@@ -1729,7 +1734,8 @@ int pccl_hip_probe_mix(const void* const* reads, int nr, void* const* writes, in
   const char* what = "pccl_hip_probe_mix";
   if (nr < 0 || nw < 0 || nr > kMaxSeg || nw > kMaxSeg || nr + nw < 1)
     return fail(PCCL_HIP_EINVAL, "%s: need 0 <= nr, nw <= %d and nr + nw >= 1", what, kMaxSeg);
-  if (shape != 0 && shape != 1) return fail(PCCL_HIP_EINVAL, "%s: shape must be 0 (one workgroup, all streams) or 1 (one stream per workgroup)", what);
+  if (shape < 0 || shape > 3)
+    return fail(PCCL_HIP_EINVAL, "%s: shape must be 0 (a workgroup serves all streams), 1 (one stream per workgroup), or 2 / 3 (the same with one-wave workgroups)", what);
   if (vectors != 1 && vectors != 2 && vectors != 4) return fail(PCCL_HIP_EINVAL, "%s: vectors per thread must be 1, 2 or 4", what);
   if (nbytes < 4096 || (nbytes & 15u)) return fail(PCCL_HIP_EINVAL, "%s: streams must hold a multiple of 16 and at least 4096 bytes", what);
   if (nr) if (int rc = check_table(reads, nr, what, "reads")) return rc;
@@ -1738,17 +1744,28 @@ int pccl_hip_probe_mix(const void* const* reads, int nr, void* const* writes, in
   for (int q = 0; q < nr; ++q) { if (!is16(reads[q])) return fail(PCCL_HIP_EINVAL, "%s: reads[%d] is not 16-byte aligned", what, q); args.rd[q] = reads[q]; }
   for (int q = 0; q < nw; ++q) { if (!is16(writes[q])) return fail(PCCL_HIP_EINVAL, "%s: writes[%d] is not 16-byte aligned", what, q); args.wr[q] = writes[q]; }
   const size_t nvec = nbytes / 16;
-  const size_t per_tile = (size_t)kThreads * (size_t)vectors;
+  const int threads = shape >= 2 ? kRowThreads : kThreads;
+  const size_t per_tile = (size_t)threads * (size_t)vectors;
   size_t tiles = (nvec + per_tile - 1) / per_tile;
-  if (shape == 1) tiles *= (size_t)(nr + nw);
+  if (shape & 1) tiles *= (size_t)(nr + nw);
   if (tiles > kMaxGrid) return fail(PCCL_HIP_EINVAL, "%s: streams too long for one launch", what);
   hipStream_t st = (hipStream_t)stream;
   const unsigned grid = (unsigned)tiles;
-  switch (vectors) {
-    case 1: PCCL_LAUNCH((k_probe_mix<1, true, true>), dim3(grid), dim3(kThreads), 0, st, args, nr, nw, nvec, shape, 0x3f803f80u); break;
-    case 2: PCCL_LAUNCH((k_probe_mix<2, true, true>), dim3(grid), dim3(kThreads), 0, st, args, nr, nw, nvec, shape, 0x3f803f80u); break;
-    default: PCCL_LAUNCH((k_probe_mix<4, true, true>), dim3(grid), dim3(kThreads), 0, st, args, nr, nw, nvec, shape, 0x3f803f80u); break;
+#define PCCL_MIX(UV, TV) PCCL_LAUNCH((k_probe_mix<UV, true, true, TV>), dim3(grid), dim3(TV), 0, st, args, nr, nw, nvec, shape, 0x3f803f80u)
+  if (threads == kRowThreads) {
+    switch (vectors) {
+      case 1: PCCL_MIX(1, kRowThreads); break;
+      case 2: PCCL_MIX(2, kRowThreads); break;
+      default: PCCL_MIX(4, kRowThreads); break;
+    }
+  } else {
+    switch (vectors) {
+      case 1: PCCL_MIX(1, kThreads); break;
+      case 2: PCCL_MIX(2, kThreads); break;
+      default: PCCL_MIX(4, kThreads); break;
+    }
   }
+#undef PCCL_MIX
   g_launches.fetch_add(1, std::memory_order_relaxed);
   return launch_status(what);
 }

@@ -724,13 +724,13 @@ __global__ __launch_bounds__(kThreads) void k_block_transpose(uint8_t* dst, cons
 // write stream with the same access shape as the kernels above.  The read
 // probe folds its data with xor and stores only if the result hits a value
 // that zero-filled or random buffers never produce, so the loads stay live.
-template <int U, bool NTL>
-__global__ __launch_bounds__(kThreads) void k_probe_read(const u32x4* src, u32x4* sink, size_t nvec) {
-  const size_t base = (size_t)blockIdx.x * (kThreads * U) + threadIdx.x;
+template <int U, bool NTL, int T = kThreads>
+__global__ __launch_bounds__(T) void k_probe_read(const u32x4* src, u32x4* sink, size_t nvec) {
+  const size_t base = (size_t)blockIdx.x * (T * U) + threadIdx.x;
   u32x4 x[U];
 #pragma unroll
   for (int j = 0; j < U; ++j) {
-    const size_t v = base + (size_t)j * kThreads;
+    const size_t v = base + (size_t)j * T;
     x[j] = v < nvec ? ld16<NTL>(src + v) : u32x4{0, 0, 0, 0};
   }
   u32x4 acc = x[0];
@@ -740,13 +740,13 @@ __global__ __launch_bounds__(kThreads) void k_probe_read(const u32x4* src, u32x4
     sink[threadIdx.x] = acc;
 }
 
-template <int U, bool NTS>
-__global__ __launch_bounds__(kThreads) void k_probe_write(u32x4* dst, size_t nvec, uint32_t value) {
-  const size_t base = (size_t)blockIdx.x * (kThreads * U) + threadIdx.x;
+template <int U, bool NTS, int T = kThreads>
+__global__ __launch_bounds__(T) void k_probe_write(u32x4* dst, size_t nvec, uint32_t value) {
+  const size_t base = (size_t)blockIdx.x * (T * U) + threadIdx.x;
   const u32x4 v4 = {value, value, value, value};
 #pragma unroll
   for (int j = 0; j < U; ++j) {
-    const size_t v = base + (size_t)j * kThreads;
+    const size_t v = base + (size_t)j * T;
     if (v < nvec) st16<NTS>(dst + v, v4);
   }
 }
@@ -762,20 +762,21 @@ struct MixArgs {
 //   shape 0: workgroup t loads tile t of every read stream and stores tile t of
 //            every write stream (the access shape of the add and fold kernels);
 //   shape 1: every workgroup serves ONE stream: workgroup w tile w / (nr + nw)
-//            of stream w % (nr + nw).
+//            of stream w % (nr + nw);
+//   shapes 2 and 3: the same two with one-wave workgroups (T = 64).
 // Loads are folded with xor and stored only on a value random data never hits.
-template <int U, bool NTL, bool NTS>
-__global__ __launch_bounds__(kThreads) void k_probe_mix(MixArgs t, int nr, int nw, size_t nvec, int shape,
+template <int U, bool NTL, bool NTS, int T = kThreads>
+__global__ __launch_bounds__(T) void k_probe_mix(MixArgs t, int nr, int nw, size_t nvec, int shape,
                                                        uint32_t value) {
   const u32x4 v4 = {value, value, value, value};
   u32x4 acc = {0, 0, 0, 0};
-  if (shape == 0) {
-    const size_t base = (size_t)blockIdx.x * (kThreads * U) + threadIdx.x;
+  if ((shape & 1) == 0) {
+    const size_t base = (size_t)blockIdx.x * (T * U) + threadIdx.x;
     for (int q = 0; q < nr; ++q) {
       u32x4 x[U];
 #pragma unroll
       for (int j = 0; j < U; ++j) {
-        const size_t v = base + (size_t)j * kThreads;
+        const size_t v = base + (size_t)j * T;
         x[j] = v < nvec ? ld16<NTL>((const u32x4*)t.rd[q] + v) : u32x4{0, 0, 0, 0};
       }
 #pragma unroll
@@ -784,19 +785,19 @@ __global__ __launch_bounds__(kThreads) void k_probe_mix(MixArgs t, int nr, int n
     for (int q = 0; q < nw; ++q) {
 #pragma unroll
       for (int j = 0; j < U; ++j) {
-        const size_t v = base + (size_t)j * kThreads;
+        const size_t v = base + (size_t)j * T;
         if (v < nvec) st16<NTS>((u32x4*)t.wr[q] + v, v4);
       }
     }
   } else {
     const unsigned streams = (unsigned)(nr + nw);
     const unsigned sidx = blockIdx.x % streams;
-    const size_t base = (size_t)(blockIdx.x / streams) * (kThreads * U) + threadIdx.x;
+    const size_t base = (size_t)(blockIdx.x / streams) * (T * U) + threadIdx.x;
     if (sidx < (unsigned)nr) {
       u32x4 x[U];
 #pragma unroll
       for (int j = 0; j < U; ++j) {
-        const size_t v = base + (size_t)j * kThreads;
+        const size_t v = base + (size_t)j * T;
         x[j] = v < nvec ? ld16<NTL>((const u32x4*)t.rd[sidx] + v) : u32x4{0, 0, 0, 0};
       }
 #pragma unroll
@@ -804,7 +805,7 @@ __global__ __launch_bounds__(kThreads) void k_probe_mix(MixArgs t, int nr, int n
     } else {
 #pragma unroll
       for (int j = 0; j < U; ++j) {
-        const size_t v = base + (size_t)j * kThreads;
+        const size_t v = base + (size_t)j * T;
         if (v < nvec) st16<NTS>((u32x4*)t.wr[sidx - nr] + v, v4);
       }
     }

@@ -30,6 +30,26 @@ def ptr(a, shift=0):
 
 
 checked = 0
+# the fused reduce with one-wave workgroups and loads in pairs (what streams from HBM get), and the general add
+# kernels on aligned data (add_rows = 0): forced here, on exact-size buffers
+lib.set_tuning("wg_kway", 64); lib.set_tuning("nt_load", 1); lib.set_tuning("nt_store", 1); lib.set_tuning("add_rows", 0)
+for dtype, code in ((O.F32, 0), (O.BF16, 1)):
+    for P in (2, 3, 4, 8, 16):
+        for B in (1, 7, 64, 1024, 4099):
+            for alg in ("ring", "recursive"):
+                if alg == "recursive" and P & (P - 1):
+                    continue
+                ins = [arr(P * B, dtype) for _ in range(P)]
+                want = (O.ring_reduce_scatter if alg == "ring" else O.recursive_halving_reduce_scatter)(ins, dtype)
+                for mode in (0, 1):
+                    outs = [np.zeros(B, ins[0].dtype) for _ in range(P)]
+                    work = [np.zeros(P * B, ins[0].dtype) for _ in range(P)]
+                    lib.reduce_scatter_virtual([ptr(o) for o in outs], [ptr(i) for i in ins],
+                                               [ptr(w) for w in work], B, code, alg, mode)
+                    for r in range(P):
+                        assert np.array_equal(outs[r].view(np.uint8), want[r].view(np.uint8)), (dtype, P, B, alg, mode)
+                    checked += 1
+lib.set_tuning("wg_kway", -1); lib.set_tuning("nt_load", -1); lib.set_tuning("nt_store", -1); lib.set_tuning("add_rows", 1)
 for unroll in (1, 4, 8):
     lib.set_tuning("unroll", unroll)
     for dtype, code in ((O.F32, 0), (O.BF16, 1)):
@@ -155,9 +175,10 @@ for alg, P, B in (("ring", 8, 4099), ("recursive", 4, 515), ("ring", 3, 1)):
 # the measurement probes on exact-size buffers
 for nb in (4096, 4096 * 5 + 16, 70000 // 16 * 16):
     bufs = [np.zeros(nb, np.uint8) for _ in range(4)]
-    lib.probe_stream(0, ptr(bufs[0]), nb)
-    lib.probe_stream(1, ptr(bufs[1]), nb)
-    for shape in (0, 1):
+    if nb >= 16384:
+        lib.probe_stream(0, ptr(bufs[0]), nb)
+        lib.probe_stream(1, ptr(bufs[1]), nb)
+    for shape in (0, 1, 2, 3):
         for vec in (1, 2, 4):
             lib.probe_mix([ptr(bufs[0]), ptr(bufs[1])], [ptr(bufs[2]), ptr(bufs[3])], nb, shape, vec)
             lib.probe_mix([ptr(bufs[0])], [], nb, shape, vec)
