@@ -565,6 +565,27 @@ def run_row(name, mode, step, info, steps, warmup, lib, verify=True):
     return row, roof, dev_ms, wall_ms, launched
 
 
+def _stream_gbps(fn, nbytes, steps, warmup):
+    """GB/s of `fn` moving nbytes per call: `warmup` untimed calls and at least WARM_MS of
+    them (see time_steps), then `steps` calls between two events."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t_warm = time.perf_counter()
+    while (time.perf_counter() - t_warm) * 1e3 < WARM_MS:
+        for _ in range(max(1, warmup)):
+            fn()
+        torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(steps):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return round(nbytes / (s.elapsed_time(e) / steps * 1e-3) / 1e9, 1)
+
+
 def ceilings(steps, warmup, device):
     """GB/s of pure read, pure write, copy and add streams over 1 GiB buffers, and
     of read:write mixes with no data flowing from the loads to the stores."""
@@ -578,16 +599,7 @@ def ceilings(steps, warmup, device):
     fa, fb, fc = (t.view(torch.float32) for t in (a, b, c))
 
     def gbps(fn, nbytes):
-        for _ in range(warmup):
-            fn()
-        torch.cuda.synchronize()
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        s.record()
-        for _ in range(steps):
-            fn()
-        e.record()
-        torch.cuda.synchronize()
-        return round(nbytes / (s.elapsed_time(e) / steps * 1e-3) / 1e9, 1)
+        return _stream_gbps(fn, nbytes, steps, warmup)
 
     st = kernels.stream_handle()
     res = {
@@ -640,16 +652,7 @@ def size_sweep(steps, warmup, device):
     from pccl import _native, kernels
 
     def gbps(fn, nbytes):
-        for _ in range(warmup):
-            fn()
-        torch.cuda.synchronize()
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        s.record()
-        for _ in range(steps):
-            fn()
-        e.record()
-        torch.cuda.synchronize()
-        return round(nbytes / (s.elapsed_time(e) / steps * 1e-3) / 1e9, 1)
+        return _stream_gbps(fn, nbytes, steps, warmup)
 
     rows = []
     for mib in (64, 128, 256, 512, 1024, 2048):

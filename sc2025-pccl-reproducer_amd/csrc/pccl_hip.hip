@@ -476,18 +476,25 @@ struct KwayLaunch {
 // narrow the window each of the k streams has in flight.  Only the one-wave
 // workgroups that streams from HBM get are limited; operands that fit the caches
 // (the footprint rule of the non-temporal hints) and 256-thread workgroups run
-// at full occupancy.  8 KiB leave 20 waves on a CU, 11 KiB 14, 16 KiB 10; 32
-// without.  Measured on MI355X (fraction of 8 TB/s at 32 / 20 / 16 / 14 waves per
-// CU): ring order, 8 bf16 shards 0.79 / 0.835 / 0.80 / 0.745, 16 bf16 shards
-// 0.77 / 0.81 / 0.81 / 0.765, 64 bf16 shards 0.76 / 0.79 / 0.79 / 0.77, 32 fp32
-// shards 0.76 / 0.81 / 0.82 / 0.84; halving order, 8 bf16 and 16 fp32 shards
-// 0.76 / 0.785 / 0.79 / 0.80, 64 bf16 shards of 1 GiB 0.79 / 0.81 / - / 0.855.
-// Launches below 512 MiB of traffic are too short to profit.
+// at full occupancy, and launches below 512 MiB of traffic are too short to
+// profit.  7 KiB leave 22 waves on a CU, 8 KiB 20, 9 KiB 17, 10 KiB 16, 11 KiB 14,
+// 12 KiB 13; 32 without.  Measured on MI355X, ring order with loads in pairs,
+// fraction of 8 TB/s at the best setting against no limit:
+//   bf16   4 shards 0.84 at 6-7 KiB (0.81)    8 shards 0.835 at 8 KiB (0.79)
+//         16 shards 0.82 at 9 KiB (0.77)      32 shards 0.80 at 9-10 KiB (0.76)
+//   fp32   4 shards 0.795 up to 10 KiB alike  8 shards 0.83 at 9-10 KiB (0.78)
+//         16 shards 0.83 at 11 KiB (0.76)     32 shards 0.84 at 11-12 KiB (0.76)
+// One KiB more per doubling of the shards, one more for fp32; a setting one step
+// off costs 1-2 %, two steps off 3-10 %.  Halving order (butterfly in
+// registers): 8 bf16 and 16 fp32 shards 0.80 at 11 KiB (0.76); its 64-way kernel
+// holds 168 registers per lane, which bounds a CU to 12 waves by itself.
 long kway_lds_pad(int k, int g, int dtype, int order, size_t traffic, int threads) {
   (void)g;
   if (threads != kRowThreads || !stream_hint(-1, traffic) || traffic < ((size_t)512 << 20)) return 0;
-  if (order == PCCL_HIP_ORDER_RING) return dtype == PCCL_HIP_F32 && k >= 24 ? 11264 : 8192;
-  return 11264;
+  if (order != PCCL_HIP_ORDER_RING) return 11264;
+  int doublings = 0;
+  while ((1 << doublings) < k) ++doublings;
+  return 5120 + 1024 * (long)doublings + (dtype == PCCL_HIP_F32 ? 1024 : 0);
 }
 
 // g = size of the inner groups of a two-level ring order (g >= k: one level).
