@@ -55,12 +55,17 @@ extern "C" {
  * PCCL_HIP_MAX_RANKS ranks goes out as several launches. */
 #define PCCL_HIP_MAX_VIRTUAL_RANKS 4096
 
-/* Element types.  bf16 sums are computed as RNE_bf16(float(a) + float(b)) at
- * every hop, which is what torch.add does on bfloat16 tensors in the
- * reference's Python algorithms (pccl/reduce_scatter.py:24,83,95,106,158). */
+/* Element types.  bf16 and fp16 sums are computed as RNE(float(a) + float(b))
+ * at every hop, which is what torch.add does on bfloat16 and float16 tensors
+ * in the reference's Python algorithms (pccl/reduce_scatter.py:24,83,95,106,158;
+ * float16 is what ZeRO hands them through pccl/patch_deepspeed.py:42-59).  The
+ * reference's compiled extension takes float32 only (pccl/src/pccl.cpp:42-45).
+ * NaN results are stored as the canonical quiet NaN of the type (0x7FC0,
+ * 0x7E00), as the host conversions of c10 do for bfloat16. */
 enum pccl_hip_dtype {
   PCCL_HIP_F32 = 0,
-  PCCL_HIP_BF16 = 1
+  PCCL_HIP_BF16 = 1,
+  PCCL_HIP_F16 = 2
 };
 
 /* Summation orders for the fused reduce (bit-exact replay of a schedule). */

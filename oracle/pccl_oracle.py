@@ -11,8 +11,8 @@ buffer of the step, then deliver", which is what simultaneous blocking
 Sendrecvs guarantee.  The schedules follow the reference line by line:
 
   vector_add                          pccl/src/common.cu:5-10 (fp32);
-                                      torch.add on bf16 tensors for bf16
-                                      (pccl/reduce_scatter.py:24,83,95,158)
+                                      torch.add on bf16 / fp16 tensors for the
+                                      16-bit types (pccl/reduce_scatter.py:24,83,95,158)
   ring_reduce_scatter                 pccl/src/reduce_scatter.cpp:101-155,
                                       pccl/reduce_scatter.py:102-161
   recursive_halving_reduce_scatter    pccl/src/reduce_scatter.cpp:16-99,
@@ -27,12 +27,13 @@ Sendrecvs guarantee.  The schedules follow the reference line by line:
   reduce_scatter_2d / all_gather_2d   pccl/reduce_scatter.py:205-235,
                                       pccl/all_gather.py:136-159
 
-Data types: "f32" arrays are numpy float32; "bf16" arrays are numpy uint16
-holding the bfloat16 bit patterns.
+Data types: "f32" arrays are numpy float32; "bf16" and "f16" arrays are numpy
+uint16 holding the bfloat16 / binary16 bit patterns.
 
 Pinning (see tests/test_oracle.py): the fp32 add is numpy's IEEE binary32 add;
 the bf16 add is checked against torch's CPU bfloat16 add over every exponent
-pair and against an independent integer rounding; the schedules are checked
+pair and against an independent integer rounding; the f16 add against torch's CPU
+float16 add over all 65 536 patterns and against the exactly rounded float64 sum; the schedules are checked
 against closed-form summation orders (left fold from rank j+1, XOR butterfly;
 for the 2-D collectives the inner order inside every node, then the outer order
 across the nodes), against exact integer sums, against P = 2 reducing to one add, against the C
@@ -45,6 +46,7 @@ import numpy as np
 
 F32 = "f32"
 BF16 = "bf16"
+F16 = "f16"
 
 
 # --------------------------------------------------------------------------
@@ -70,11 +72,28 @@ def f32_to_bf16(x: np.ndarray) -> np.ndarray:
     return np.where(np.isnan(x), np.uint16(0x7FC0), rounded).astype(np.uint16)
 
 
+def f16_to_f32(u: np.ndarray) -> np.ndarray:
+    """Widen binary16 bit patterns (uint16) to float32: exact."""
+    return np.ascontiguousarray(u, dtype=np.uint16).view(np.float16).astype(np.float32)
+
+
+def f32_to_f16(x: np.ndarray) -> np.ndarray:
+    """Round float32 to binary16 bit patterns, round-to-nearest-even (numpy's
+    conversion; values beyond 65504 + half an ulp become infinity).  NaN maps to
+    the canonical quiet NaN 0x7E00."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    with np.errstate(over="ignore", invalid="ignore"):
+        h = x.astype(np.float16).view(np.uint16)
+    return np.where(np.isnan(x), np.uint16(0x7E00), h).astype(np.uint16)
+
+
 def vector_add(a: np.ndarray, b: np.ndarray, dtype: str) -> np.ndarray:
     """a[i] + b[i] in the arithmetic of `dtype` (one hop of any schedule).
 
     f32: one IEEE-754 binary32 RNE add (pccl/src/common.cu:8).
-    bf16: RNE_bf16(float(a) + float(b)), the fp32 sum itself RNE."""
+    bf16: RNE_bf16(float(a) + float(b)), the fp32 sum itself RNE.
+    f16:  RNE_f16(float(a) + float(b)); binary32 has 24 >= 2*11+2 significand
+          bits, so this is the correctly rounded binary16 sum."""
     if dtype == F32:
         with np.errstate(over="ignore", invalid="ignore"):
             return (np.asarray(a, np.float32) + np.asarray(b, np.float32)).astype(np.float32)
@@ -82,6 +101,10 @@ def vector_add(a: np.ndarray, b: np.ndarray, dtype: str) -> np.ndarray:
         with np.errstate(over="ignore", invalid="ignore"):
             s = bf16_to_f32(a) + bf16_to_f32(b)
         return f32_to_bf16(s)
+    if dtype == F16:
+        with np.errstate(over="ignore", invalid="ignore"):
+            s = f16_to_f32(a) + f16_to_f32(b)
+        return f32_to_f16(s)
     raise ValueError(f"unknown dtype {dtype!r}")
 
 

@@ -38,7 +38,7 @@ def parse_args(argv=None):
     parser.add_argument("--test", action="store_true", help="test for correctness")
     parser.add_argument("--pccl-recursive-alg", action="store_true",
                         help="Use the recursive doubling algorithm for PCCL.")
-    parser.add_argument("--dtype", choices=["fp32", "bf16"], default="fp32")
+    parser.add_argument("--dtype", choices=["fp32", "bf16", "fp16"], default="fp32")
     parser.add_argument("--world-size", type=int, default=None,
                         help="number of virtual ranks (default: $SLURM_NTASKS or 8)")
     parser.add_argument("--sizes", type=int, nargs="*", default=None, help="output sizes per rank in MB")
@@ -62,7 +62,7 @@ def main(argv=None):
     sizes = np.array(args.sizes if args.sizes else [1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024])
     unit = "MB"
     use_rd = args.pccl_recursive_alg
-    dtype = torch.float32 if args.dtype == "fp32" else torch.bfloat16
+    dtype = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[args.dtype]
     esize = 4 if args.dtype == "fp32" else 2
     library = args.library
     if library == "pccl":

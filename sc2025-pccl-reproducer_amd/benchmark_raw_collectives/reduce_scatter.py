@@ -43,7 +43,7 @@ def parse_args(argv=None):
     parser.add_argument("--test", action="store_true", help="test for correctness")
     parser.add_argument("--pccl-recursive-alg", action="store_true",
                         help="Use the recursive halving algorithm for PCCL.")
-    parser.add_argument("--dtype", choices=["fp32", "bf16"], default="fp32")
+    parser.add_argument("--dtype", choices=["fp32", "bf16", "fp16"], default="fp32")
     parser.add_argument("--world-size", type=int, default=None,
                         help="number of virtual ranks (default: $SLURM_NTASKS or 8)")
     parser.add_argument("--sizes", type=int, nargs="*", default=None, help="input sizes per rank in MB")
@@ -67,7 +67,7 @@ def main(argv=None):
     sizes = np.array(args.sizes if args.sizes else [1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024])
     unit = "MB"
     use_rh = args.pccl_recursive_alg
-    dtype = torch.float32 if args.dtype == "fp32" else torch.bfloat16
+    dtype = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[args.dtype]
     esize = 4 if args.dtype == "fp32" else 2
     library = args.library
     if library == "pccl":
@@ -114,8 +114,9 @@ def main(argv=None):
                 for t in inputs:
                     gold += t.float()
                 hops = world_size - 1
+                ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11      # one rounding per hop
                 tol = dict(rtol=1e-5, atol=1e-8) if dtype == torch.float32 else \
-                    dict(rtol=hops * 2.0 ** -8, atol=hops * 2.0 ** -8 * float(gold.abs().mean()))
+                    dict(rtol=hops * ulp, atol=hops * ulp * float(gold.abs().mean()))
                 for r in range(world_size):
                     assert allclose(outputs[r].float(), gold[r * output_numel:(r + 1) * output_numel], **tol)
 

@@ -211,7 +211,7 @@ void with_tuning(const Tune& t, F&& f) {
 }
 
 size_t esize_of(int dtype) {
-  return dtype == PCCL_HIP_F32 ? 4 : dtype == PCCL_HIP_BF16 ? 2 : 0;
+  return dtype == PCCL_HIP_F32 ? 4 : (dtype == PCCL_HIP_BF16 || dtype == PCCL_HIP_F16) ? 2 : 0;
 }
 
 Pieces contiguous(size_t n) {
@@ -234,8 +234,10 @@ struct AddLaunch {
     for_spans((size_t)count * pc.s1 * pc.s2 * tiles, [&](Span span, unsigned grid) {
       if (dtype == PCCL_HIP_F32)
         PCCL_LAUNCH((k_add_segs<OpF32, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *segs, count, pc, tiles, aligned, span);
-      else
+      else if (dtype == PCCL_HIP_BF16)
         PCCL_LAUNCH((k_add_segs<OpBF16, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *segs, count, pc, tiles, aligned, span);
+      else
+        PCCL_LAUNCH((k_add_segs<OpF16, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *segs, count, pc, tiles, aligned, span);
     });
   }
   template <int U, bool NTL, bool NTS>
@@ -255,9 +257,12 @@ void launch_add_rows(const AddSegs& segs, int count, size_t n, int dtype, const 
     if (dtype == PCCL_HIP_F32) {
       if (t.ntl) { if (t.nts) PCCL_ROWS(OpF32, true, true); else PCCL_ROWS(OpF32, true, false); }
       else { if (t.nts) PCCL_ROWS(OpF32, false, true); else PCCL_ROWS(OpF32, false, false); }
-    } else {
+    } else if (dtype == PCCL_HIP_BF16) {
       if (t.ntl) { if (t.nts) PCCL_ROWS(OpBF16, true, true); else PCCL_ROWS(OpBF16, true, false); }
       else { if (t.nts) PCCL_ROWS(OpBF16, false, true); else PCCL_ROWS(OpBF16, false, false); }
+    } else {
+      if (t.ntl) { if (t.nts) PCCL_ROWS(OpF16, true, true); else PCCL_ROWS(OpF16, true, false); }
+      else { if (t.nts) PCCL_ROWS(OpF16, false, true); else PCCL_ROWS(OpF16, false, false); }
     }
 #undef PCCL_ROWS
     g_launches.fetch_add(1, std::memory_order_relaxed);
@@ -380,8 +385,10 @@ struct RhLaunch {
     for_spans((size_t)P * tiles, [&](Span span, unsigned grid) {
       if (dtype == PCCL_HIP_F32)
         PCCL_LAUNCH((k_rh_round<OpF32, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *args, P, B, round, from_src, to_outs, tiles, aligned, span);
-      else
+      else if (dtype == PCCL_HIP_BF16)
         PCCL_LAUNCH((k_rh_round<OpBF16, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *args, P, B, round, from_src, to_outs, tiles, aligned, span);
+      else
+        PCCL_LAUNCH((k_rh_round<OpF16, U, NTL, NTS, T>), dim3(grid), dim3(T), lds, stream, *args, P, B, round, from_src, to_outs, tiles, aligned, span);
     });
   }
   template <int U, bool NTL, bool NTS>
@@ -466,8 +473,10 @@ struct KwayLaunch {
   void operator()() const {
     constexpr int UK = 1;
     if (dtype == PCCL_HIP_F32) run<AccF32, UK, NTL, NTS>();
-    else if (per_hop) run<AccBF16<true>, UK, NTL, NTS>();
-    else run<AccBF16<false>, UK, NTL, NTS>();
+    else if (dtype == PCCL_HIP_BF16 && per_hop) run<AccBF16<true>, UK, NTL, NTS>();
+    else if (dtype == PCCL_HIP_BF16) run<AccBF16<false>, UK, NTL, NTS>();
+    else if (per_hop) run<AccF16<true>, UK, NTL, NTS>();
+    else run<AccF16<false>, UK, NTL, NTS>();
   }
 };
 
@@ -662,7 +671,7 @@ int check_table(const void* const* tab, int count, const char* what, const char*
 
 int check_dtype(int dtype, const char* what) {
   if (esize_of(dtype) == 0)
-    return fail(PCCL_HIP_EINVAL, "%s: unknown dtype %d (0 = float32, 1 = bfloat16)", what, dtype);
+    return fail(PCCL_HIP_EINVAL, "%s: unknown dtype %d (0 = float32, 1 = bfloat16, 2 = float16)", what, dtype);
   return PCCL_HIP_OK;
 }
 
@@ -832,9 +841,12 @@ int pccl_hip_rh_round(void* const* bufs, const void* const* src, void* const* ou
       if (dtype == PCCL_HIP_F32) {
         if (t.ntl) { if (t.nts) PCCL_RH(OpF32, true, true); else PCCL_RH(OpF32, true, false); }
         else { if (t.nts) PCCL_RH(OpF32, false, true); else PCCL_RH(OpF32, false, false); }
-      } else {
+      } else if (dtype == PCCL_HIP_BF16) {
         if (t.ntl) { if (t.nts) PCCL_RH(OpBF16, true, true); else PCCL_RH(OpBF16, true, false); }
         else { if (t.nts) PCCL_RH(OpBF16, false, true); else PCCL_RH(OpBF16, false, false); }
+      } else {
+        if (t.ntl) { if (t.nts) PCCL_RH(OpF16, true, true); else PCCL_RH(OpF16, true, false); }
+        else { if (t.nts) PCCL_RH(OpF16, false, true); else PCCL_RH(OpF16, false, false); }
       }
 #undef PCCL_RH
       g_launches.fetch_add(1, std::memory_order_relaxed);

@@ -135,6 +135,47 @@ struct OpBF16 {
   }
 };
 
+// binary16 <-> binary32.  Widening is exact; narrowing rounds to nearest even
+// (v_cvt_f16_f32), and NaN becomes the canonical 0x7E00.  An fp16 hop is
+// RNE_fp16(float(a) + float(b)), what torch.add does on float16 tensors on the
+// host; since binary32 carries 24 >= 2 * 11 + 2 significand bits, rounding the
+// fp32 sum once more gives the correctly rounded fp16 sum.
+__device__ __forceinline__ float f16_widen(uint32_t u16) {
+  const uint16_t u = (uint16_t)u16;
+  _Float16 h;
+  __builtin_memcpy(&h, &u, 2);
+  return (float)h;
+}
+
+__device__ __forceinline__ uint32_t f16_narrow(float s) {
+  const _Float16 h = (_Float16)s;
+  uint16_t u;
+  __builtin_memcpy(&u, &h, 2);
+  return (s != s) ? 0x7e00u : (uint32_t)u;
+}
+
+// Two fp16 values per 32-bit word, element 2i in the low half.
+struct OpF16 {
+  typedef uint16_t elem;
+  static constexpr int kPerVec = 8;
+  static __device__ __forceinline__ uint32_t add_word(uint32_t a, uint32_t b) {
+    const float lo = f16_widen(a & 0xffffu) + f16_widen(b & 0xffffu);
+    const float hi = f16_widen(a >> 16) + f16_widen(b >> 16);
+    return f16_narrow(lo) | (f16_narrow(hi) << 16);
+  }
+  static __device__ __forceinline__ u32x4 add(u32x4 a, u32x4 b) {
+    u32x4 r;
+    r.x = add_word(a.x, b.x);
+    r.y = add_word(a.y, b.y);
+    r.z = add_word(a.z, b.z);
+    r.w = add_word(a.w, b.w);
+    return r;
+  }
+  static __device__ __forceinline__ elem add1(elem a, elem b) {
+    return (elem)f16_narrow(f16_widen(a) + f16_widen(b));
+  }
+};
+
 // Partial sums of the fused reduce.  An accumulator is held as fp32 lanes; for
 // bf16 with per-hop rounding the fp32 value is re-rounded to bf16 precision
 // after every add, which is bit-identical to storing and re-loading bf16.
@@ -145,6 +186,8 @@ struct AccF32 {
     f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y);
     f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
   }
+  static __device__ __forceinline__ float widen1(float e) { return e; }
+  static __device__ __forceinline__ float narrow1(float f) { return f; }
   static __device__ __forceinline__ float hop(float a, float b) { return a + b; }
   // one hop of a ring: the running sum `acc` is what the rank received, x its own block
   template <int L>
@@ -180,6 +223,8 @@ struct AccBF16 {
     f[4] = __uint_as_float(v.z << 16); f[5] = __uint_as_float(v.z & 0xffff0000u);
     f[6] = __uint_as_float(v.w << 16); f[7] = __uint_as_float(v.w & 0xffff0000u);
   }
+  static __device__ __forceinline__ float widen1(uint16_t e) { return __uint_as_float((uint32_t)e << 16); }
+  static __device__ __forceinline__ uint16_t narrow1(float f) { return (uint16_t)(bf16_round_hi(f) >> 16); }
   static __device__ __forceinline__ float hop(float a, float b) {
     float s = a + b;
     if constexpr (PER_HOP) return __uint_as_float(bf16_round_hi(s));
@@ -231,6 +276,45 @@ struct AccBF16 {
     widen(v, f);
     return narrow(f);
   }
+};
+
+template <bool PER_HOP>
+struct AccF16 {
+  typedef OpF16 op;
+  static constexpr int kLanes = 8;
+  static __device__ __forceinline__ void widen(u32x4 v, float* f) {
+    f[0] = f16_widen(v.x & 0xffffu); f[1] = f16_widen(v.x >> 16);
+    f[2] = f16_widen(v.y & 0xffffu); f[3] = f16_widen(v.y >> 16);
+    f[4] = f16_widen(v.z & 0xffffu); f[5] = f16_widen(v.z >> 16);
+    f[6] = f16_widen(v.w & 0xffffu); f[7] = f16_widen(v.w >> 16);
+  }
+  static __device__ __forceinline__ float widen1(uint16_t e) { return f16_widen(e); }
+  static __device__ __forceinline__ uint16_t narrow1(float f) { return (uint16_t)f16_narrow(f); }
+  static __device__ __forceinline__ float hop(float a, float b) {
+    const float s = a + b;
+    if constexpr (PER_HOP) return f16_widen(f16_narrow(s));
+    else return s;
+  }
+  template <int L>
+  static __device__ __forceinline__ void hop_lanes(float* acc, const float* x) {
+#pragma unroll
+    for (int l = 0; l < L; ++l) acc[l] = hop(acc[l], x[l]);
+  }
+  // NaNs are stored as the canonical pattern, so the two operands' roles do not matter here
+  template <int L>
+  static __device__ __forceinline__ void join_lanes(float* lo, const float* hi) { hop_lanes<L>(lo, hi); }
+  static __device__ __forceinline__ u32x4 narrow(const float* f) {
+    u32x4 r;
+    r.x = f16_narrow(f[0]) | (f16_narrow(f[1]) << 16);
+    r.y = f16_narrow(f[2]) | (f16_narrow(f[3]) << 16);
+    r.z = f16_narrow(f[4]) | (f16_narrow(f[5]) << 16);
+    r.w = f16_narrow(f[6]) | (f16_narrow(f[7]) << 16);
+    return r;
+  }
+  // with a rounding per hop every partial sum is an fp16 value again and can stay packed
+  static constexpr bool kPacked = PER_HOP;
+  static __device__ __forceinline__ u32x4 add_vec(u32x4 a, u32x4 b) { return OpF16::add(a, b); }
+  static __device__ __forceinline__ u32x4 settle(u32x4 v) { return v; }   // OpF16::add stores canonical NaNs already
 };
 
 // How a segment of `n` elements splits into a head (elements before the first
@@ -1042,12 +1126,10 @@ __global__ __launch_bounds__(T) void k_reduce_kway(KwayArgs t, int k, int g, int
             if constexpr (K > 0) asm volatile("" : "+s"(q));   // fetch the pointer here, see group_load
 #endif
             elem e = ((const elem*)t.shard[q] + eoff)[i];
-            if constexpr (sizeof(elem) == 4) f[0] = e;
-            else f[0] = __uint_as_float((uint32_t)e << 16);
+            f[0] = Acc::widen1(e);
           },
           k, g, first, first_outer, acc1);
-      if constexpr (sizeof(elem) == 4) out[i] = acc1[0];
-      else out[i] = (elem)(bf16_round_hi(acc1[0]) >> 16);
+      out[i] = Acc::narrow1(acc1[0]);
     }
   }
 }

@@ -17,6 +17,7 @@ from typing import Optional, Sequence
 
 F32 = 0
 BF16 = 1
+F16 = 2
 
 ORDER_RING = 0
 ORDER_HALVING = 1

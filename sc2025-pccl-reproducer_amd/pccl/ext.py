@@ -9,9 +9,9 @@ collective (include/pccl_hip.h: pccl_hip_reduce_scatter_virtual /
 pccl_hip_all_gather_virtual).  Like the reference they return None with the
 work queued on the current stream.
 
-Deviation kept on purpose: reduce_scatter accepts bfloat16 as well as float32
-(the reference's extension rejects everything but float, pccl.cpp:42-45; its
-Python algorithms are what run bf16).
+Deviation kept on purpose: reduce_scatter accepts bfloat16 and float16 as well as
+float32 (the reference's extension rejects everything but float, pccl.cpp:42-45;
+its Python algorithms are what run the 16-bit types).
 """
 from __future__ import annotations
 
@@ -45,7 +45,7 @@ def reduce_scatter_mpi(output_tensor: torch.Tensor, input_tensor: torch.Tensor, 
     block_size = total_elems // size
     if output_tensor.numel() != block_size:
         raise RuntimeError("Output tensor must have block_size elements (input tensor numel()/world_size)")
-    if input_tensor.dtype not in (torch.float32, torch.bfloat16):
+    if input_tensor.dtype not in (torch.float32, torch.bfloat16, torch.float16):
         raise RuntimeError("Input tensor must be of type float")
     if output_tensor.dtype != input_tensor.dtype:
         raise RuntimeError("Output tensor must be of type float")

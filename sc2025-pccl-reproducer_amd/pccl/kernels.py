@@ -14,7 +14,7 @@ from typing import List, Optional, Sequence
 import torch
 
 from . import _native
-from ._native import (BF16, F32, MODE_FAITHFUL, MODE_FUSED, MODE_STEPS, ORDER_HALVING,
+from ._native import (BF16, F16, F32, MODE_FAITHFUL, MODE_FUSED, MODE_STEPS, ORDER_HALVING,
                       ORDER_RING, MAX_RANKS, MAX_VIRTUAL_RANKS)
 
 _MODES = {"steps": MODE_STEPS, "fused": MODE_FUSED, "faithful": MODE_FAITHFUL}
@@ -43,13 +43,15 @@ def mode_code(mode) -> int:
 
 def dtype_code(dtype: torch.dtype) -> int:
     """Element type of the reduction kernels.  The reference's extension takes
-    float32 only (pccl/src/pccl.cpp:42-45); bfloat16 is what its Python
-    algorithms add with torch.add."""
+    float32 only (pccl/src/pccl.cpp:42-45); bfloat16 and float16 are what its
+    Python algorithms add with torch.add (pccl/reduce_scatter.py:24,83,95,158)."""
     if dtype == torch.float32:
         return F32
     if dtype == torch.bfloat16:
         return BF16
-    raise RuntimeError("Input tensor must be of type float (float32 or bfloat16)")
+    if dtype == torch.float16:
+        return F16
+    raise RuntimeError("Input tensor must be of type float (float32, bfloat16 or float16)")
 
 
 # the raw handle of torch's current stream without building a Stream object (a

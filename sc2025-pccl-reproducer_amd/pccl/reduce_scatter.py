@@ -30,7 +30,7 @@ from .virtual import VirtualComm
 def _reduce_into(dst: torch.Tensor, recv: torch.Tensor, op):
     """dst = op(dst, recv).  torch.add maps onto the accumulate kernel
     (pccl/src/common.cu:5-19); any other callable is applied as given."""
-    if op is torch.add and dst.dtype in (torch.float32, torch.bfloat16):
+    if op is torch.add and dst.dtype in (torch.float32, torch.bfloat16, torch.float16):
         kernels.accumulate(dst, recv)
     else:
         dst.copy_(op(dst, recv))

@@ -18,7 +18,7 @@ def make_inputs(P, n, dtype, seed=0, dist="normal", scale=1.0):
             x = rng.integers(-8, 9, n).astype(np.float32)
         else:
             raise ValueError(dist)
-        out.append(x if dtype == O.F32 else O.f32_to_bf16(x))
+        out.append(x if dtype == O.F32 else O.f32_to_bf16(x) if dtype == O.BF16 else O.f32_to_f16(x))
     return out
 
 
@@ -27,7 +27,7 @@ def to_torch(x, dtype, device):
     x = np.array(x, copy=True)            # never share memory with the oracle's inputs
     if dtype == O.F32:
         return torch.from_numpy(x).to(device)
-    return torch.from_numpy(x.view(np.int16)).to(device).view(torch.bfloat16)
+    return torch.from_numpy(x.view(np.int16)).to(device).view(torch.bfloat16 if dtype == O.BF16 else torch.float16)
 
 
 def to_numpy(t, dtype):

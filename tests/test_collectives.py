@@ -14,7 +14,7 @@ MODES = ["steps", "fused", "faithful"]
 
 def _tdtype(dtype):
     import torch
-    return torch.float32 if dtype == O.F32 else torch.bfloat16
+    return {O.F32: torch.float32, O.BF16: torch.bfloat16, O.F16: torch.float16}[dtype]
 
 
 def _rs_oracle(alg):

@@ -435,3 +435,72 @@ def test_oracle_reproduces_golden_vectors(path):
             assert_bits_equal(z[f"out_{r}"], np.concatenate(ins), "fixture vs concatenation")
     for r in range(P):
         assert_bits_equal(outs[r], z[f"out_{r}"], f"rank {r}")
+
+
+# ---- binary16 ---------------------------------------------------------------------
+
+def _f16_partners():
+    return np.concatenate([np.arange(0, 65536, 1024, dtype=np.uint16) | np.uint16(0x135),
+                           np.array([0x0000, 0x8000, 0x7C00, 0xFC00, 0x0001, 0x8001, 0x03FF, 0x0400, 0x7BFF, 0xFBFF,
+                                     0x3C00, 0x3C01, 0x7E00, 0x7D01], np.uint16)])
+
+
+def test_f16_add_is_torch_add():
+    """The hop arithmetic of the reference's Python algorithms on float16 tensors
+    (pccl/reduce_scatter.py:24,83,95,158): torch.add, all 65 536 patterns against
+    78 partners (every exponent, zeros, infinities, subnormals, the largest finite
+    values, NaNs)."""
+    import torch
+    a = np.arange(65536, dtype=np.uint16)
+    partners = _f16_partners()
+    A, B = np.tile(a, partners.size), np.repeat(partners, a.size)
+    ta = torch.from_numpy(A.view(np.int16).copy()).view(torch.float16)
+    tb = torch.from_numpy(B.view(np.int16).copy()).view(torch.float16)
+    want = torch.add(ta, tb).view(torch.int16).numpy().view(np.uint16)
+    got = O.vector_add(A, B, O.F16)
+    nan = np.isnan(want.view(np.float16))
+    assert nan.any() and (~nan).sum() > 4_000_000
+    assert np.array_equal(got[~nan], want[~nan])
+    assert (got[nan] == 0x7E00).all()                 # the oracle stores the canonical quiet NaN
+
+
+def test_f16_add_is_the_correctly_rounded_sum():
+    """float64 holds the sum of two binary16 values exactly; rounding it ONCE to
+    binary16 (nearest even) must give the oracle's result, which rounds twice
+    (to binary32, then to binary16): 24 >= 2 * 11 + 2 bits make that harmless.
+    Rounding toward zero instead gives other bits (the check has teeth)."""
+    a = np.arange(65536, dtype=np.uint16)
+    partners = _f16_partners()
+    A, B = np.tile(a, partners.size), np.repeat(partners, a.size)
+    with np.errstate(over="ignore", invalid="ignore"):
+        exact = A.view(np.float16).astype(np.float64) + B.view(np.float16).astype(np.float64)
+        want = exact.astype(np.float16).view(np.uint16)
+    got = O.vector_add(A, B, O.F16)
+    ok = ~np.isnan(exact)
+    assert np.array_equal(got[ok], want[ok])
+    with np.errstate(over="ignore", invalid="ignore"):
+        toward_zero = np.where(np.abs(want.view(np.float16).astype(np.float64)) > np.abs(exact),
+                               want - np.uint16(1), want)
+    assert (toward_zero[ok] != got[ok]).sum() > 100_000
+
+
+def test_f16_conversions_round_trip_and_saturate_to_infinity():
+    u = np.arange(65536, dtype=np.uint16)
+    f = O.f16_to_f32(u)
+    back = O.f32_to_f16(f)
+    nan = np.isnan(f)
+    assert np.array_equal(back[~nan], u[~nan]) and (back[nan] == 0x7E00).all()
+    assert O.f32_to_f16(np.array([65504.0, 65519.9, 65520.0, -65520.0, 1e-8, 5.96e-8], np.float32)).tolist() == \
+        [0x7BFF, 0x7BFF, 0x7C00, 0xFC00, 0x0000, 0x0001]
+
+
+@pytest.mark.parametrize("alg", ["ring", "recursive"])
+def test_f16_schedules_follow_the_closed_forms(alg):
+    P, B = 8, 257
+    ins = make_inputs(P, P * B, O.F16, seed=40)
+    if alg == "ring":
+        got, want = O.ring_reduce_scatter(ins, O.F16), ring_closed_form(ins, O.F16)
+    else:
+        got, want = O.recursive_halving_reduce_scatter(ins, O.F16), halving_closed_form(ins, O.F16)
+    for r in range(P):
+        assert_bits_equal(got[r], want[r], f"rank {r}")
