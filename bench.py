@@ -21,6 +21,7 @@ Workloads:
   cfg1  ring reduce_scatter, P=4, fp32, 16 Mi elements per rank
   cfg2  ring reduce_scatter, P=8, bf16, 256 Mi elements per rank, per-hop
         accumulate with bf16 rounding at every hop
+  cfg2h the cfg2 shape in float16 (the third element type; no BASELINE row)
   cfg3  recursive-halving round at its largest shape: a pair of ranks adding
         512 MiB strided halves (bf16), i.e. round 0 of P=64 with 1 GiB per rank
   cfg3full  the whole recursive-halving reduce_scatter over P=64 resident ranks,
@@ -61,9 +62,9 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
 MiB = 1 << 20
 WARM_MS = 60.0               # least duration of the untimed warm-up before a timed region, see time_steps
 
-WORKLOADS = ["cfg1", "cfg2", "cfg3", "cfg3full", "cfg4", "cfg4u", "cfg5"]
+WORKLOADS = ["cfg1", "cfg2", "cfg2h", "cfg3", "cfg3full", "cfg4", "cfg4u", "cfg5"]
 # every (workload, mode) row of the default run besides the headline cfg2/steps
-ALL_ROWS = [("cfg1", "steps"), ("cfg1", "fused"), ("cfg2", "fused"), ("cfg3", "steps"),
+ALL_ROWS = [("cfg1", "steps"), ("cfg1", "fused"), ("cfg2", "fused"), ("cfg2h", "steps"), ("cfg2h", "fused"), ("cfg3", "steps"),
             ("cfg3full", "steps"), ("cfg3full", "fused"), ("cfg4", "steps"), ("cfg4", "fused"),
             ("cfg4u", "fused"), ("cfg5", "fused"), ("cfg5", "steps")]
 
@@ -98,16 +99,16 @@ def parse_args():
 # resident on the GPU
 # ---------------------------------------------------------------------------
 
-def _randn_bf16(n, std, seed, device, out=None):
+def _randn_bf16(n, std, seed, device, out=None, dtype=None):
     import torch
     g = torch.Generator(device=device)
     g.manual_seed(seed)
     if out is None:
-        out = torch.empty(n, dtype=torch.bfloat16, device=device)
+        out = torch.empty(n, dtype=dtype or torch.bfloat16, device=device)
     chunk = 1 << 26
     for i in range(0, n, chunk):      # bounded fp32 temporaries
         m = min(chunk, n - i)
-        out[i:i + m] = (torch.randn(m, generator=g, device=device) * std).to(torch.bfloat16)
+        out[i:i + m] = (torch.randn(m, generator=g, device=device) * std).to(out.dtype)
     return out
 
 
@@ -161,14 +162,14 @@ def _hop(acc, x):
     """One hop of the reference's accumulate on torch tensors: an IEEE fp32 add,
     rounded to bfloat16 (nearest even) when the data is bfloat16."""
     import torch
-    if acc.dtype == torch.bfloat16:
-        return (acc.float() + x.float()).to(torch.bfloat16)
+    if acc.dtype in (torch.bfloat16, torch.float16):
+        return (acc.float() + x.float()).to(acc.dtype)
     return acc + x
 
 
 def _same_bits(a, b):
     import torch
-    it = torch.int16 if a.dtype == torch.bfloat16 else torch.int32
+    it = torch.int32 if a.dtype == torch.float32 else torch.int16
     return torch.equal(a.view(it), b.view(it))
 
 
@@ -177,14 +178,14 @@ def make_ring_rs(P, elems_per_rank, dtype, modes, device, seed=1234, std=1.0):
     from pccl import kernels
     B = elems_per_rank // P
     total = B * P
-    tdt = torch.bfloat16 if dtype == "bf16" else torch.float32
+    tdt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dtype]
     ins = _slab(P, total, tdt, device)
     for r in range(P):
-        if dtype == "bf16":
+        if dtype in ("bf16", "f16"):
             _randn_bf16(total, std, seed + r, device, out=ins[r])
         else:
             _rand_f32(total, seed + r, device, out=ins[r])
-    es = 2 if dtype == "bf16" else 4
+    es = 4 if dtype == "f32" else 2
     outs = _slab(P, B, tdt, device)
     shared = {}
 
@@ -451,6 +452,8 @@ def build_workloads(name, modes, scale, device):
         return make_ring_rs(4, sc(16 * MiB), "f32", modes, device)
     if name == "cfg2":
         return make_ring_rs(8, sc(256 * MiB), "bf16", modes, device, std=1e-2)
+    if name == "cfg2h":
+        return make_ring_rs(8, sc(256 * MiB), "f16", modes, device, std=1e-2)
     if name == "cfg3":
         pair = make_rh_pair(sc(256 * MiB), device)
         return {m: pair["steps"] for m in modes}

@@ -493,8 +493,9 @@ struct KwayLaunch {
 //         16 shards 0.82 at 9 KiB (0.77)      32 shards 0.80 at 9-10 KiB (0.76)
 //   fp32   4 shards 0.795 up to 10 KiB alike  8 shards 0.83 at 9-10 KiB (0.78)
 //         16 shards 0.83 at 11 KiB (0.76)     32 shards 0.84 at 11-12 KiB (0.76)
-// One KiB more per doubling of the shards, one more for fp32; a setting one step
-// off costs 1-2 %, two steps off 3-10 %.  Halving order (butterfly in
+//   fp16   8 shards 0.845 at 7 KiB (0.78; 0.81 at 8 KiB)
+// One KiB more per doubling of the shards, one more for fp32, one less for fp16; a
+// setting one step off costs 1-4 %, two steps off 3-10 %.  Halving order (butterfly in
 // registers): 8 bf16 and 16 fp32 shards 0.80 at 11 KiB (0.76); its 64-way kernel
 // holds 168 registers per lane, which bounds a CU to 12 waves by itself.
 long kway_lds_pad(int k, int g, int dtype, int order, size_t traffic, int threads) {
@@ -503,7 +504,7 @@ long kway_lds_pad(int k, int g, int dtype, int order, size_t traffic, int thread
   if (order != PCCL_HIP_ORDER_RING) return 11264;
   int doublings = 0;
   while ((1 << doublings) < k) ++doublings;
-  return 5120 + 1024 * (long)doublings + (dtype == PCCL_HIP_F32 ? 1024 : 0);
+  return 5120 + 1024 * (long)doublings + (dtype == PCCL_HIP_F32 ? 1024 : dtype == PCCL_HIP_F16 ? -1024 : 0);
 }
 
 // g = size of the inner groups of a two-level ring order (g >= k: one level).
