@@ -49,7 +49,7 @@ def test_counter_traffic_is_tied_to_the_kernel_sources(monkeypatch):
     lib = _Tuning(dict(table["tuning"]))
     got, why = bench.profiled_traffic("cfg2", "steps", "k_add_rows", lib, 1.0)
     assert why is None and got == table["entries"]["cfg2:steps:k_add_rows"]
-    assert abs(got / (3 * 8 * (32 << 20) * 2 / 2) - 1) < 0.01          # ~ the algorithmic bytes of one launch
+    assert abs(got / (3 * 8 * (32 << 20) * 2) - 1) < 0.01              # ~ the algorithmic bytes of one launch (= one step)
     # another size, another tuning, an unknown row, other sources: no figure, and the reason
     assert bench.profiled_traffic("cfg2", "steps", "k_add_rows", lib, 0.5)[0] is None
     other = _Tuning(dict(table["tuning"], unroll=8))
