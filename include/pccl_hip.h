@@ -376,7 +376,8 @@ int pccl_hip_set_tuning(const char* key, long value);
 long pccl_hip_get_tuning(const char* key);
 
 /* Kernel launches this process has issued through the library so far (a step
- * of a schedule may be several, see "launch_mib").  For measurement: the
+ * of a schedule is one launch up to 64 ranks and one per 64 ranks beyond; a
+ * fused collective is one or a few, see the entry points).  For measurement: the
  * difference around a timed region is the number of launches in it.  No
  * counterpart in the reference. */
 unsigned long long pccl_hip_launch_count(void);
