@@ -22,6 +22,9 @@ Workloads:
   cfg2  ring reduce_scatter, P=8, bf16, 256 Mi elements per rank, per-hop
         accumulate with bf16 rounding at every hop
   cfg2h the cfg2 shape in float16 (the third element type; no BASELINE row)
+  cfg2d reduce_scatter_2D of the cfg2 data on a grid of 2 nodes x 4 local ranks, ring on
+        both levels, as one fused launch (what the reference's harness runs with
+        --library pccl; no BASELINE row)
   cfg3  recursive-halving round at its largest shape: a pair of ranks adding
         512 MiB strided halves (bf16), i.e. round 0 of P=64 with 1 GiB per rank
   cfg3full  the whole recursive-halving reduce_scatter over P=64 resident ranks,
@@ -62,9 +65,10 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
 MiB = 1 << 20
 WARM_MS = 60.0               # least duration of the untimed warm-up before a timed region, see time_steps
 
-WORKLOADS = ["cfg1", "cfg2", "cfg2h", "cfg3", "cfg3full", "cfg4", "cfg4u", "cfg5"]
+WORKLOADS = ["cfg1", "cfg2", "cfg2h", "cfg2d", "cfg3", "cfg3full", "cfg4", "cfg4u", "cfg5"]
 # every (workload, mode) row of the default run besides the headline cfg2/steps
-ALL_ROWS = [("cfg1", "steps"), ("cfg1", "fused"), ("cfg2", "fused"), ("cfg2h", "steps"), ("cfg2h", "fused"), ("cfg3", "steps"),
+ALL_ROWS = [("cfg1", "steps"), ("cfg1", "fused"), ("cfg2", "fused"), ("cfg2h", "steps"), ("cfg2h", "fused"), ("cfg2d", "fused"),
+            ("cfg3", "steps"),
             ("cfg3full", "steps"), ("cfg3full", "fused"), ("cfg4", "steps"), ("cfg4", "fused"),
             ("cfg4u", "fused"), ("cfg5", "fused"), ("cfg5", "steps")]
 
@@ -228,6 +232,63 @@ def make_ring_rs(P, elems_per_rank, dtype, modes, device, seed=1234, std=1.0):
                  f"({total * es / MiB:.0f} MiB), block {B} elements, mode={_mode_name(m)}",
             dtype=dtype, P=P, B=B, verify=verify,
             verify_how="left fold from rank j+1 recomputed with torch on windows of blocks 0, P/2, P-1"))
+    return out
+
+
+def make_grid_rs(intra, inter, elems_per_rank, dtype, modes, device, seed=4321, std=1e-2):
+    """reduce_scatter_2D (pccl/reduce_scatter.py:205-235) over a grid of inter nodes x intra
+    local ranks, ring order on both levels, as ONE fused launch: what the reference's
+    benchmark harness runs with --library pccl."""
+    import torch
+    from pccl import kernels
+    W = intra * inter
+    m = elems_per_rank // W
+    total = m * W
+    tdt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dtype]
+    es = 4 if dtype == "f32" else 2
+    ins = _slab(W, total, tdt, device)
+    for r in range(W):
+        if dtype == "f32":
+            _rand_f32(total, seed + r, device, out=ins[r])
+        else:
+            _randn_bf16(total, std, seed + r, device, out=ins[r])
+    outs = _slab(W, m, tdt, device)
+
+    def ring_fold(parts, j):
+        acc = parts[(j + 1) % len(parts)]
+        for t in range(2, len(parts) + 1):
+            acc = _hop(acc, parts[(j + t) % len(parts)])
+        return acc
+
+    def verify():
+        # rank w = node * intra + local ends with block w: first the ring order of block `local` over the
+        # locals of every node, then the ring order of block `node` over the nodes, one rounding per hop
+        torch.cuda.synchronize()
+        for w in sorted({0, W // 2, W - 1}):
+            node, local = divmod(w, intra)
+            for lo, hi in _windows(m):
+                per_node = [ring_fold([ins[n * intra + l][w * m + lo:w * m + hi] for l in range(intra)], local)
+                            for n in range(inter)]
+                if not _same_bits(outs[w][lo:hi], ring_fold(per_node, node)):
+                    return False
+        return True
+
+    out = {}
+    for mode in modes:
+        if kernels.mode_code(mode) != kernels.MODE_FUSED:
+            raise ValueError("the 2-D workload is measured in the fused mode")
+
+        def step():
+            kernels.reduce_scatter_2d_ranks(outs, ins, intra, inter, "ring", "fused")
+
+        nbytes = (W * W + W) * m * es
+        out[mode] = (step, dict(
+            alg_bytes=nbytes, kernel="k_reduce_kway", kernel_bytes=nbytes, kernel_launches=1, launches=1,
+            desc=f"reduce_scatter_2D, {inter} nodes x {intra} local ranks (virtual), ring on both levels, {dtype}, "
+                 f"{total} elements per rank ({total * es / MiB:.0f} MiB), block {m} elements, mode=fused",
+            dtype=dtype, P=W, B=m, verify=verify,
+            verify_how="two-level left fold (locals from local+1, then nodes from node+1) recomputed with torch on "
+                       "windows of blocks 0, W/2, W-1"))
     return out
 
 
@@ -440,7 +501,7 @@ def make_kway(k, n, modes, device, seed=11):
 
 
 def default_mode(name):
-    return "fused" if name in ("cfg4", "cfg4u", "cfg5") else "steps"
+    return "fused" if name in ("cfg2d", "cfg4", "cfg4u", "cfg5") else "steps"
 
 
 def build_workloads(name, modes, scale, device):
@@ -454,6 +515,8 @@ def build_workloads(name, modes, scale, device):
         return make_ring_rs(8, sc(256 * MiB), "bf16", modes, device, std=1e-2)
     if name == "cfg2h":
         return make_ring_rs(8, sc(256 * MiB), "f16", modes, device, std=1e-2)
+    if name == "cfg2d":
+        return make_grid_rs(4, 2, sc(256 * MiB), "bf16", modes, device)
     if name == "cfg3":
         pair = make_rh_pair(sc(256 * MiB), device)
         return {m: pair["steps"] for m in modes}
@@ -645,7 +708,9 @@ def ceilings(steps, warmup, device):
         mixes[f"{nr}r{nw}w_{mib}MiB"] = {"probe": best, "probe_shape": shape, "library_kernel": kname,
                                          "library": mine, "library_over_probe": round(mine / best, 3)}
         del rd, wr
-    res["mixes"] = mixes
+    res["reference_mixes"] = mixes
+    res["reference_mixes_note"] = ("dependence-free probes of the same read:write mix: reference points, not bounds "
+                                   "(a ratio above 1 = the library kernel orders its work better than the probe's plain shapes)")
     return res
 
 

@@ -495,16 +495,25 @@ struct KwayLaunch {
 //         16 shards 0.83 at 11 KiB (0.76)     32 shards 0.84 at 11-12 KiB (0.76)
 //   fp16   8 shards 0.845 at 7 KiB (0.78; 0.81 at 8 KiB)
 // One KiB more per doubling of the shards, one more for fp32, one less for fp16; a
-// setting one step off costs 1-4 %, two steps off 3-10 %.  Halving order (butterfly in
-// registers): 8 bf16 and 16 fp32 shards 0.80 at 11 KiB (0.76); its 64-way kernel
-// holds 168 registers per lane, which bounds a CU to 12 waves by itself.
+// setting one step off costs 1-4 %, two steps off 3-10 %.  Beyond 32 shards the
+// best setting falls back to that of 16 (64 shards: bf16 0.785 at 8-9 KiB, fp32
+// 0.79 at 9-10 KiB, against 0.76 and 0.775 at 11 KiB).  The two-level ring order of
+// the 2-D collectives issues its loads in chains of g shards (one inner group at a
+// time), wants more waves for it, and follows g instead of k, without the extra KiB
+// for fp32: best settings 4x2 bf16 7 KiB (0.815; 0.77 at 8 KiB), 2x4 6 KiB (0.81;
+// 0.69 at 8 KiB), 4x4 7 KiB, 8x8 8 KiB, 16x4 9-10 KiB; fp32 2x4 6 KiB (0.83), 4x2 and
+// 4x4 7 KiB (0.84, 0.81), 8x8 8-10 KiB; fp16 4x2 and 4x4 6 KiB.  Halving order
+// (butterfly in registers): 8 bf16 and 16 fp32 shards 0.80 at 11 KiB (0.76); its
+// 64-way kernel holds 168 registers per lane, which bounds a CU to 12 waves by itself.
 long kway_lds_pad(int k, int g, int dtype, int order, size_t traffic, int threads) {
-  (void)g;
   if (threads != kRowThreads || !stream_hint(-1, traffic) || traffic < ((size_t)512 << 20)) return 0;
   if (order != PCCL_HIP_ORDER_RING) return 11264;
+  const bool two_level = g < k;
+  const int chain = two_level ? g : k > 32 ? 16 : k;
   int doublings = 0;
-  while ((1 << doublings) < k) ++doublings;
-  return 5120 + 1024 * (long)doublings + (dtype == PCCL_HIP_F32 ? 1024 : dtype == PCCL_HIP_F16 ? -1024 : 0);
+  while ((1 << doublings) < chain) ++doublings;
+  const long by_type = dtype == PCCL_HIP_F16 ? -1024 : (dtype == PCCL_HIP_F32 && !two_level) ? 1024 : 0;
+  return 5120 + 1024 * (long)doublings + by_type;
 }
 
 // g = size of the inner groups of a two-level ring order (g >= k: one level).
@@ -609,11 +618,13 @@ class ExtentList {
   int check(const char* what) {
     Extent* v = big_.empty() ? small_ : big_.data();
     std::sort(v, v + n_, [](const Extent& a, const Extent& b) { return a.lo != b.lo ? a.lo < b.lo : a.kind < b.kind; });
-    // sweep by start address; `top` is the started extent that reaches farthest
-    // among the writers and among the readers, `partner` the one reader a writer
-    // may coincide with (or the one writer a reader may lie in)
+    // sweep by start address; `topw` is the started writer that reaches farthest (writers
+    // never overlap each other, so it is the only one that can still be open), `topr` and
+    // `nextr` the two started readers that reach farthest: a writer may start inside ONE
+    // reader, its partner, so no other reader may reach to where it starts
     const Extent* topw = nullptr;
     const Extent* topr = nullptr;
+    const Extent* nextr = nullptr;
     for (size_t i = 0; i < n_; ++i) {
       const Extent& x = v[i];
       const bool xw = x.kind != 'i';
@@ -626,12 +637,15 @@ class ExtentList {
         const Extent& r = *topr;
         const bool ok = x.in_place && x.kind == 'o' && r.rank == x.rank && pairs(r, x);
         if (!ok) return clash(what, r, x);
-        // no second reader may reach into it either: the readers that started before the top one
-        for (size_t j = 0; j < i; ++j)
-          if (v[j].kind == 'i' && &v[j] != topr && v[j].hi > x.lo) return clash(what, v[j], x);
+        if (nextr && nextr->hi > x.lo) return clash(what, *nextr, x);
       }
-      if (xw) { if (!topw || x.hi > topw->hi) topw = &x; }
-      else { if (!topr || x.hi > topr->hi) topr = &x; }
+      if (xw) {
+        if (!topw || x.hi > topw->hi) topw = &x;
+      } else if (!topr || x.hi > topr->hi) {
+        nextr = topr; topr = &x;
+      } else if (!nextr || x.hi > nextr->hi) {
+        nextr = &x;
+      }
     }
     return PCCL_HIP_OK;
   }
@@ -1440,7 +1454,8 @@ int pccl_hip_reduce_scatter_2d_virtual(void* const* outputs, const void* const* 
     if (ring) {
       // world order; block w of every input; inner ring inside each node, then the ring across nodes
       for (int w = 0; w < W; ++w) { args.shard[w] = inputs[w]; args.out[w] = outputs[w]; args.eoff[w] = (size_t)w * m; }
-      return launch_kway(args, W, inter == 1 ? W : intra, W, m, dtype, PCCL_HIP_ORDER_RING, 1, 1, st, what);
+      // (one rank per node, or one node: the flat ring, whose loads go out in pairs)
+      return launch_kway(args, W, (inter == 1 || intra == 1) ? W : intra, W, m, dtype, PCCL_HIP_ORDER_RING, 1, 1, st, what);
     }
     // halving inside the node, then across nodes = ONE butterfly over the index
     // q = i*inter + j (inner bits above outer bits), rooted at the output's own q

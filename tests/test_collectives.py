@@ -786,6 +786,11 @@ def test_overlapping_buffers_are_refused(target):
     refused([big[P * B - 8:][:B]] + t_out[1:], t_in, "faithful", [big[:P * B]] + work[1:])
     # inputs may share memory among themselves
     kernels.reduce_scatter_ranks(t_out, [t_in[0]] * P, "ring", "fused")
+    # ... but an output that is in place in its own input must not lie in a second input as well,
+    # whichever of the two aliased inputs comes first in the table
+    refused([t_in[0][0:B]] + t_out[1:], [t_in[0], t_in[0]] + t_in[2:], "fused")
+    refused([t_out[0], t_in[1][B:2 * B]] + t_out[2:], [t_in[1]] + t_in[1:], "steps", work)
+    refused(t_out[:3] + [t_in[3][3 * B:]], t_in[:2] + [t_in[3], t_in[3]], "fused")
     # all_gather: a shard inside another rank's output, outputs on top of each other
     g_out = [torch.zeros(P * B, device=dev) for _ in range(P)]
     g_in = [torch.zeros(B, device=dev) for _ in range(P)]
