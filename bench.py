@@ -94,7 +94,7 @@ def parse_args():
                          "FETCH_SIZE / WRITE_SIZE readings scale the hardware counters of a rocprofv3 --pmc run")
     ap.add_argument("--tune", action="append", default=[], metavar="KEY=VALUE",
                     help="launch tuning of the library: any key of pccl_hip_set_tuning (grid_cap, unroll, unroll_copy, "
-                         "nt_load, nt_store, add_rows, wg_kway, lds_pad_*, gather_strip, gather_split, unroll_gather, gather_nt)")
+                         "nt_load, nt_store, add_rows, fold_rows, wg_kway, lds_pad_*, gather_strip, gather_split, unroll_gather, gather_nt)")
     return ap.parse_args()
 
 
@@ -220,7 +220,8 @@ def make_ring_rs(P, elems_per_rank, dtype, modes, device, seed=1234, std=1.0):
         if m == kernels.MODE_FUSED:
             kernel_bytes = (P * P + P) * B * es             # reads every input once, writes every output
             alg_bytes = kernel_bytes
-            kernel = "k_reduce_kway"
+            # aligned ring folds over at most 16 fp32 / bf16 shards run in the lean kernel
+            kernel = "k_fold_rows" if P <= 16 and dtype in ("bf16", "f32") else "k_reduce_kway"
         else:
             kernel_bytes = 3 * P * B * es                   # one batched step: 2 reads + 1 write per rank
             alg_bytes = (P - 1) * kernel_bytes
@@ -697,7 +698,8 @@ def ceilings(steps, warmup, device):
         if nw == 1 and nr == 2:
             mine, kname = gbps(lambda: kernels.add(wr[0], rd[0], rd[1]), 3 * nb), "k_add_rows"
         elif nw == 1:
-            mine, kname = gbps(lambda: kernels.reduce_kway(wr[0], rd, "ring", 1), (nr + 1) * nb), "k_reduce_kway"
+            mine, kname = gbps(lambda: kernels.reduce_kway(wr[0], rd, "ring", 1), (nr + 1) * nb), \
+                "k_fold_rows" if nr <= 16 else "k_reduce_kway"
         else:
             # nw shards of nb / nw bytes into nw outputs of nb bytes: nb read, nw * nb written
             g_out = [w.view(torch.uint8) for w in wr]
@@ -977,7 +979,7 @@ def cpu_baseline(info):
             subprocess.run(["make", "-C", os.path.join(ROOT, "oracle")], check=True, capture_output=True)
         except Exception as e:                               # noqa: BLE001
             return {"value": None, "unit": "GB/s", "cores": 0, "kind": "port", "sample": f"not built: {e}"}
-    P = info["P"] if info["kernel"] in ("k_add_rows", "k_add_segs", "k_reduce_kway") and info["P"] <= 8 else 8
+    P = info["P"] if info["kernel"] in ("k_add_rows", "k_add_segs", "k_reduce_kway", "k_fold_rows") and info["P"] <= 8 else 8
     dtype = "bf16" if info["dtype"] == "bf16" else "f32"
     host_cores = os.cpu_count() or 1
     ranks = min(P, max(1, host_cores))
@@ -1019,7 +1021,7 @@ def cpu_baseline(info):
 
 # ---------------------------------------------------------------------------
 
-TUNING_KEYS = ("grid_cap", "unroll", "add_rows", "wg_kway", "unroll_copy", "nt_load", "nt_store", "gather_strip",
+TUNING_KEYS = ("grid_cap", "unroll", "add_rows", "fold_rows", "wg_kway", "unroll_copy", "nt_load", "nt_store", "gather_strip",
                "gather_split", "unroll_gather", "gather_nt", "lds_pad_copy", "lds_pad_kway",
                "lds_pad_gather")
 

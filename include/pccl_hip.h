@@ -337,6 +337,10 @@ int pccl_hip_probe_mix(const void* const* reads, int nr, void* const* writes,
  *      "add_rows" (1, the default: adds over contiguous 16-byte aligned
  *                  segments run in the lean one-wave kernels, one 128-bit
  *                  vector per thread; 0: everything in the general kernels),
+ *      "fold_rows" (1, the default: a ring-order fused reduce over at most 16
+ *                  fp32 or bfloat16 shards that streams from HBM, with every
+ *                  operand 16-byte aligned, runs in the lean kernel on a 2-D
+ *                  grid; 0: always the general kernel),
  *      "unroll"   (128-bit vectors per thread per operand of the general add
  *                  kernels: 1, 2, 4 or 8), "unroll_copy" (the same for the copy
  *                  kernels),

@@ -17,6 +17,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <type_traits>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -80,6 +81,7 @@ std::atomic<long> g_unroll_copy{2};   // ... copy kernels (two 4 KiB chunks per 
 // window the chip streams from at any moment.  0 = as many as fit (8).
 std::atomic<long> g_lds_pad_copy{-1};  // copy kernels; -1 = chosen per launch (see copy_lds_pad)
 std::atomic<long> g_lds_pad_kway{-1};  // fused reduce; -1 = chosen per launch (see launch_kway)
+std::atomic<long> g_fold_rows{1};      // aligned folds of streams from HBM go to the lean kernel (k_fold_rows); 0 = always the general kernel
 std::atomic<long> g_wg_kway{-1};       // threads per workgroup of the fused reduce: 64, 256, or -1 = 64 for streams from HBM
 std::atomic<long> g_lds_pad_gather{-1}; // all_gather placement kernels; -1 = chosen per launch
 std::atomic<long> g_gather_split{0};   // groups of outputs per shard tile in the multicast gather; 0 = four outputs a group
@@ -439,6 +441,7 @@ struct KwayLaunch {
   size_t n, tiles;
   unsigned lds_pad;
   int threads;
+  bool rows;
   hipStream_t stream;
 
   template <class Acc, int U, bool NTL, bool NTS, int T, int PF>
@@ -460,10 +463,22 @@ struct KwayLaunch {
 #undef PCCL_KWAY
   }
 
+  // ring order; every output, shard and element offset 16-byte aligned, whole vectors: the lean kernel on a 2-D grid
+  template <class Acc>
+  void run_rows() const {
+    const size_t nvec = n * sizeof(typename Acc::op::elem) / 16;
+    const dim3 grid((unsigned)((nvec + kRowThreads - 1) / kRowThreads), (unsigned)nout);
+    PCCL_LAUNCH((k_fold_rows<Acc, 0, true, true, 2>), grid, dim3(kRowThreads), lds_pad, stream, *args, k, g, first0, nvec);
+    g_launches.fetch_add(1, std::memory_order_relaxed);
+  }
+
   template <class Acc, int U, bool NTL, bool NTS>
   void run() const {
     if constexpr (NTL && NTS) {
       // streams from HBM: one-wave workgroups, ring-order loads in pairs whatever k, one launch
+      if constexpr (!std::is_same<Acc, AccF16<true>>::value && !std::is_same<Acc, AccF16<false>>::value) {
+        if (threads == kRowThreads && rows) { run_rows<Acc>(); return; }
+      }
       if (threads == kRowThreads) { run_wg<Acc, U, NTL, NTS, kRowThreads, 2>(); return; }
     }
     run_wg<Acc, U, NTL, NTS, kThreads, kFoldPairedFrom>();
@@ -485,35 +500,54 @@ struct KwayLaunch {
 // narrow the window each of the k streams has in flight.  Only the one-wave
 // workgroups that streams from HBM get are limited; operands that fit the caches
 // (the footprint rule of the non-temporal hints) and 256-thread workgroups run
-// at full occupancy, and launches below 512 MiB of traffic are too short to
-// profit.  7 KiB leave 22 waves on a CU, 8 KiB 20, 9 KiB 17, 10 KiB 16, 11 KiB 14,
-// 12 KiB 13; 32 without.  Measured on MI355X, ring order with loads in pairs,
-// fraction of 8 TB/s at the best setting against no limit:
-//   bf16   4 shards 0.84 at 6-7 KiB (0.81)    8 shards 0.835 at 8 KiB (0.79)
-//         16 shards 0.82 at 9 KiB (0.77)      32 shards 0.80 at 9-10 KiB (0.76)
-//   fp32   4 shards 0.795 up to 10 KiB alike  8 shards 0.83 at 9-10 KiB (0.78)
-//         16 shards 0.83 at 11 KiB (0.76)     32 shards 0.84 at 11-12 KiB (0.76)
-//   fp16   8 shards 0.845 at 7 KiB (0.78; 0.81 at 8 KiB)
-// One KiB more per doubling of the shards, one more for fp32, one less for fp16; a
-// setting one step off costs 1-4 %, two steps off 3-10 %.  Beyond 32 shards the
-// best setting falls back to that of 16 (64 shards: bf16 0.785 at 8-9 KiB, fp32
-// 0.79 at 9-10 KiB, against 0.76 and 0.775 at 11 KiB).  The two-level ring order of
-// the 2-D collectives issues its loads in chains of g shards (one inner group at a
-// time), wants more waves for it, and follows g instead of k, without the extra KiB
-// for fp32: best settings 4x2 bf16 7 KiB (0.815; 0.77 at 8 KiB), 2x4 6 KiB (0.81;
-// 0.69 at 8 KiB), 4x4 7 KiB, 8x8 8 KiB, 16x4 9-10 KiB; fp32 2x4 6 KiB (0.83), 4x2 and
-// 4x4 7 KiB (0.84, 0.81), 8x8 8-10 KiB; fp16 4x2 and 4x4 6 KiB.  Halving order
-// (butterfly in registers): 8 bf16 and 16 fp32 shards 0.80 at 11 KiB (0.76); its
-// 64-way kernel holds 168 registers per lane, which bounds a CU to 12 waves by itself.
+// at full occupancy.  6 KiB leave 26 waves on a CU, 7 KiB 22, 8 KiB 20, 9 KiB 17, 10 KiB 16,
+// 11 KiB 14, 12 KiB 13; 32 without.  Measured on MI355X, ring order with loads in
+// pairs, 512 MiB per rank, fraction of 8 TB/s at the best setting (and without a
+// limit); up to 16 shards in the lean kernel, beyond in the general one:
+//   bf16   2 shards 0.85 without (7 KiB: 0.79)    3: 0.85 at 7 KiB (0.80)
+//          4: 0.87 at 7 KiB (0.80)                 5: 0.855 at 8 KiB (0.80)
+//          6: 0.83 at 8 KiB (0.79)                 8: 0.835-0.85 at 8 KiB (0.78)
+//         12: 0.82 at 8 KiB (0.76)                16: 0.82 at 9 KiB (0.76)
+//         24: 0.80 at 9-10 KiB (0.75)             32: 0.80 at 9-10 KiB (0.76)
+//         64: 0.785 at 8-9 KiB (0.76)
+//   fp16   (general kernel) 4 shards 0.85 at 6 KiB, 8: 0.845 at 7 KiB (0.78), 16: 0.80 at 8 KiB
+//   fp32   2 and 3 shards 0.83, 0.815 without (flat up to 10 KiB for 3)
+//          4: 0.83 at 9-10 KiB (0.80)              5: 0.835 at 11 KiB (0.795)
+//          6, 8: 0.845 at 11 KiB (0.785)          12, 16: 0.82 at 11 KiB (0.76)
+//         24: 0.80 at 11 KiB (0.74)               32: 0.84 at 11-12 KiB (0.76)
+//         64: 0.79 at 9-10 KiB (0.755)
+// A setting one step off costs 1-4 %, two steps off 3-10 %.  The two-level ring
+// order of the 2-D collectives issues its loads in chains of g shards (one inner
+// group at a time), wants more waves for it, and follows g, fp32 like bf16: best
+// settings 4x2 bf16 7 KiB (0.815; 0.77 at 8 KiB), 2x4 6 KiB (0.81; 0.69 at 8 KiB),
+// 3x2 7 KiB, 4x4 7 KiB, 8x8 8 KiB, 16x4 9-10 KiB; fp32 2x4 6 KiB (0.83), 4x2 and
+// 4x4 7 KiB (0.84, 0.81), 6x2 8 KiB, 8x8 8-10 KiB; fp16 4x2 and 4x4 6 KiB.  Halving
+// order (butterfly in registers; 8 shards with their loads in pairs): 4 shards
+// bf16 0.81 at 9-10 KiB, fp16 0.815 at 9 KiB, fp32 0.83 at 8 KiB (0.80 without);
+// 8 shards bf16 0.84 and fp16 0.82 at 7 KiB, fp32 0.85 at 11 KiB (0.79); 16 fp32
+// shards 0.80 at 11 KiB (0.76); the kernels for 32 and 64 shards hold 105-182
+// registers per lane, which bounds a CU to 8-16 waves by itself.
 long kway_lds_pad(int k, int g, int dtype, int order, size_t traffic, int threads) {
-  if (threads != kRowThreads || !stream_hint(-1, traffic) || traffic < ((size_t)512 << 20)) return 0;
-  if (order != PCCL_HIP_ORDER_RING) return 11264;
-  const bool two_level = g < k;
-  const int chain = two_level ? g : k > 32 ? 16 : k;
-  int doublings = 0;
-  while ((1 << doublings) < chain) ++doublings;
-  const long by_type = dtype == PCCL_HIP_F16 ? -1024 : (dtype == PCCL_HIP_F32 && !two_level) ? 1024 : 0;
-  return 5120 + 1024 * (long)doublings + by_type;
+  if (threads != kRowThreads || !stream_hint(-1, traffic)) return 0;
+  if (k <= 2) return 0;
+  if (order != PCCL_HIP_ORDER_RING) {
+    if (traffic < ((size_t)512 << 20)) return 0;   // not measured below
+    if (k == 4) return dtype == PCCL_HIP_F32 ? 8192 : dtype == PCCL_HIP_F16 ? 9216 : 10240;
+    if (k == 8) return dtype == PCCL_HIP_F32 ? 11264 : 7168;
+    return 11264;
+  }
+  const long by_type = dtype == PCCL_HIP_F16 ? -1024 : 0;
+  if (g < k) {                           // two-level: 1 KiB per doubling of the inner group, rounded up
+    int doublings = 0;
+    while ((1 << doublings) < g) ++doublings;
+    return 5120 + 1024 * (long)doublings + by_type;
+  }
+  if (dtype == PCCL_HIP_F32) {
+    // the wide limits of fp32 cost 1-4 % on launches of 320 MiB over 4 or 8 shards and gain from 0.6 GiB on
+    if (k <= 8 && traffic < ((size_t)512 << 20)) return 0;
+    return k <= 3 ? 0 : k == 4 ? 9216 : k <= 32 ? 11264 : 10240;
+  }
+  return (k <= 4 ? 7168 : k < 16 ? 8192 : k < 32 ? 9216 : k == 32 ? 10240 : 9216) + by_type;
 }
 
 // g = size of the inner groups of a two-level ring order (g >= k: one level).
@@ -532,8 +566,16 @@ int launch_kway(const KwayArgs& args, int k, int g, int nout, size_t n, int dtyp
   if (!(tune.ntl && tune.nts)) wg = kThreads;   // the one-wave variant exists for non-temporal streams only
   long pad = g_lds_pad_kway.load(std::memory_order_relaxed);
   if (pad < 0) pad = kway_lds_pad(k, g, dtype, order, traffic, (int)wg);
+  const size_t es = esize_of(dtype);
+  // The lean kernel for what it measured faster for on MI355X: the flat ring order over up to 16 fp32 or bf16
+  // shards (+2-3 % at 4-16 shards; 32 and 64 shards, the two-level ring and the butterfly -2...0 %, float16 -1 %).
+  bool rows = wg == kRowThreads && g_fold_rows.load(std::memory_order_relaxed) && order == PCCL_HIP_ORDER_RING &&
+              g >= k && k <= 16 && dtype != PCCL_HIP_F16 && (n * es) % 16 == 0 &&
+              n * es / 16 <= (size_t)kMaxGrid * kRowThreads;
+  for (int q = 0; rows && q < k; ++q) rows = (uintptr_t)args.shard[q] % 16 == 0;
+  for (int j = 0; rows && j < nout; ++j) rows = (uintptr_t)args.out[j] % 16 == 0 && (args.eoff[j] * es) % 16 == 0;
   KwayLaunch l{&args, k, g, nout, dtype, order, first0, per_hop, n, tiles_for(n * esize_of(dtype), 1, (int)wg),
-               (unsigned)pad, (int)wg, stream};
+               (unsigned)pad, (int)wg, rows, stream};
   if (int rc = check_work_items((size_t)nout, l.tiles, what)) return rc;
   with_tuning(tune, l);
   return launch_status(what);
@@ -718,6 +760,8 @@ int pccl_hip_set_tuning(const char* key, long value) {
     g_wg_kway = value;
   } else if (!strcmp(key, "add_rows")) {
     g_add_rows = value != 0;
+  } else if (!strcmp(key, "fold_rows")) {
+    g_fold_rows = value != 0;
   } else if (!strcmp(key, "unroll_copy")) {
     if (value != 1 && value != 2 && value != 4 && value != 8)
       return fail(PCCL_HIP_EINVAL, "set_tuning: unroll_copy must be 1, 2, 4 or 8");
@@ -759,6 +803,7 @@ long pccl_hip_get_tuning(const char* key) {
   if (!strcmp(key, "unroll")) return g_unroll;
   if (!strcmp(key, "wg_kway")) return g_wg_kway;
   if (!strcmp(key, "add_rows")) return g_add_rows;
+  if (!strcmp(key, "fold_rows")) return g_fold_rows;
   if (!strcmp(key, "unroll_copy")) return g_unroll_copy;
   if (!strcmp(key, "lds_pad_copy")) return g_lds_pad_copy;
   if (!strcmp(key, "lds_pad_kway")) return g_lds_pad_kway;

@@ -209,6 +209,7 @@ struct AccF32 {
   }
   // one hop on whole input vectors: partial sums can stay in input format
   static constexpr bool kPacked = true;
+  static constexpr bool kAsmAdd = true;   // the add is an asm statement (add_own_received): loads are not hoisted over it
   static __device__ __forceinline__ u32x4 add_vec(u32x4 a, u32x4 b) { return OpF32::add(a, b); }
   static __device__ __forceinline__ u32x4 settle(u32x4 v) { return v; }
 };
@@ -260,6 +261,7 @@ struct AccBF16 {
   // With a rounding per hop every partial sum is a bf16 value again, so partial
   // sums can stay packed two to a word (half the registers of fp32 lanes).
   static constexpr bool kPacked = PER_HOP;
+  static constexpr bool kAsmAdd = false;
   static __device__ __forceinline__ uint32_t add_word(uint32_t a, uint32_t b) {
     return cvt_pk_bf16(__uint_as_float(a << 16) + __uint_as_float(b << 16),
                        __uint_as_float(a & 0xffff0000u) + __uint_as_float(b & 0xffff0000u));
@@ -313,6 +315,7 @@ struct AccF16 {
   }
   // with a rounding per hop every partial sum is an fp16 value again and can stay packed
   static constexpr bool kPacked = PER_HOP;
+  static constexpr bool kAsmAdd = false;
   static __device__ __forceinline__ u32x4 add_vec(u32x4 a, u32x4 b) { return OpF16::add(a, b); }
   static __device__ __forceinline__ u32x4 settle(u32x4 v) { return v; }   // OpF16::add stores canonical NaNs already
 };
@@ -916,7 +919,24 @@ __device__ __forceinline__ void tree_sum(Load& load, int first, float* out) {
     float lo[L], hi[L];
     tree_sum<Acc, K, M, 2 * H, L>(load, first, lo);
     tree_sum<Acc, K, M + H, 2 * H, L>(load, first, hi);
+#if defined(__HIP_DEVICE_COMPILE__)
+    // Eight shards: the two leaves of a pair are loaded together, ahead of their
+    // add, and the next pair is not loaded before this one is summed (the sum must
+    // exist at the second fence: an empty asm takes it as operand): two loads in
+    // flight per wave, as in the ring order.  Left alone, the scheduler issues 6 of
+    // the 8 loads up front for the 16-bit types and sinks every fp32 load down to
+    // its add (an asm statement); both measured 4-6 % slower on MI355X.  Four
+    // shards measured the same or slower with the fences and stay without.
+    if constexpr (2 * H == K && K == 8) __builtin_amdgcn_sched_barrier(0);
+#endif
     Acc::template join_lanes<L>(lo, hi);
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (2 * H == K && K == 8) {
+#pragma unroll
+      for (int l = 0; l < L; ++l) asm volatile("" : "+v"(lo[l]));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#endif
 #pragma unroll
     for (int l = 0; l < L; ++l) out[l] = lo[l];
   }
@@ -939,6 +959,14 @@ __device__ __forceinline__ void tree_vec(Load& load, u32x4* out) {
     u32x4 lo[G], hi[G];
     tree_vec<Acc, KG, M, 2 * H, G>(load, lo);
     tree_vec<Acc, KG, M + H, 2 * H, G>(load, hi);
+#if defined(__HIP_DEVICE_COMPILE__)
+    // 64 fp32 shards: both leaf groups are loaded ahead of their adds.  The fp32
+    // add is an asm statement, and the scheduler otherwise sinks each load down to
+    // its add: one load in flight, 0.70 of the peak on MI355X against 0.80 with the
+    // fence.  The 16-bit types do not need it, and 16 and 32 shards measured 4-6 %
+    // slower with it, whatever the type.
+    if constexpr (2 * H == KG && KG >= 8 && Acc::kAsmAdd) __builtin_amdgcn_sched_barrier(0);
+#endif
 #pragma unroll
     for (int r = 0; r < G; ++r) out[r] = Acc::add_vec(lo[r], hi[r]);
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -1037,6 +1065,45 @@ __device__ __forceinline__ void fold_shards(Load&& load, int k, int g, int first
   }
 }
 
+// One 128-bit vector of one output: the fold over the k shards at byte offset
+// wg_byte (uniform over the workgroup) + lane_byte, stored to dst.
+template <class Acc, int K, bool NTL, bool NTS, int PF>
+__device__ __forceinline__ void fold_vector(const KwayArgs& t, int k, int g, int first, int first_outer,
+                                            size_t wg_byte, uint32_t lane_byte, u32x4* dst) {
+  constexpr int L = Acc::kLanes;
+  if constexpr (K >= 16 && Acc::kPacked) {
+    constexpr int G = tree_group<K>();
+    u32x4 part[G];
+    auto group_load = [&](int b, u32x4* x) {
+#pragma unroll
+      for (int r = 0; r < G; ++r) {
+        int q = first ^ (G * b + r);
+#if defined(__HIP_DEVICE_COMPILE__)
+        // ties the fetch of the shard pointer to this place: left alone, all K
+        // pointers are fetched up front and spill out of the scalar registers
+        asm volatile("" : "+s"(q));
+#endif
+        x[r] = ld16u<NTL>((const uint8_t*)t.shard[q] + wg_byte + lane_byte);
+      }
+    };
+    tree_vec<Acc, K / G, 0, 1, G>(group_load, part);
+#pragma unroll
+    for (int h = G / 2; h >= 1; h /= 2) {
+#pragma unroll
+      for (int r = 0; r < h; ++r) part[r] = Acc::add_vec(part[r], part[r + h]);
+    }
+    st16<NTS>(dst, Acc::settle(part[0]));
+  } else {
+    float acc[L];
+    fold_shards<Acc, K, L, PF>(
+        [&](int q, float* f) {
+          Acc::widen(ld16u<NTL>((const uint8_t*)t.shard[q] + wg_byte + lane_byte), f);
+        },
+        k, g, first, first_outer, acc);
+    st16<NTS>(dst, Acc::narrow(acc));
+  }
+}
+
 // Fused k-way reduce, one pass: output j = fold over the k shards of
 // shard[.][eoff[j] + i], i < n, starting the schedule at shard
 // (first0 + j) mod k (or, for the two-level ring, at the inner and outer
@@ -1048,7 +1115,6 @@ __global__ __launch_bounds__(T) void k_reduce_kway(KwayArgs t, int k, int g, int
                                                           size_t tiles_per_seg, Span span) {
   typedef typename Acc::op Op;
   typedef typename Op::elem elem;
-  constexpr int L = Acc::kLanes;
   const uint32_t tps = (uint32_t)tiles_per_seg;
   const unsigned tid = threadIdx.x;
   for (uint64_t w64 = (uint64_t)span.begin + blockIdx.x; w64 < span.end; w64 += gridDim.x) {
@@ -1078,40 +1144,8 @@ __global__ __launch_bounds__(T) void k_reduce_kway(KwayArgs t, int k, int g, int
       // the unrolled folds then need no vector registers for their k addresses
       const size_t wg_byte = (eoff + head) * sizeof(elem) + (base + (size_t)u * T) * 16;
       const uint32_t lane_byte = tid * 16u;
-      if constexpr (K >= 16 && Acc::kPacked) {
-        if (v < nvec) {
-          constexpr int G = tree_group<K>();
-          u32x4 part[G];
-          auto group_load = [&](int b, u32x4* x) {
-#pragma unroll
-            for (int r = 0; r < G; ++r) {
-              int q = first ^ (G * b + r);
-#if defined(__HIP_DEVICE_COMPILE__)
-              // ties the fetch of the shard pointer to this place: left alone, all K
-              // pointers are fetched up front and spill out of the scalar registers
-              asm volatile("" : "+s"(q));
-#endif
-              x[r] = ld16u<NTL>((const uint8_t*)t.shard[q] + wg_byte + lane_byte);
-            }
-          };
-          tree_vec<Acc, K / G, 0, 1, G>(group_load, part);
-#pragma unroll
-          for (int h = G / 2; h >= 1; h /= 2) {
-#pragma unroll
-            for (int r = 0; r < h; ++r) part[r] = Acc::add_vec(part[r], part[r + h]);
-          }
-          st16<NTS>((u32x4*)(out + head) + v, Acc::settle(part[0]));
-        }
-      } else
-      if (v < nvec) {
-        float acc[L];
-        fold_shards<Acc, K, L, PF>(
-            [&](int q, float* f) {
-              Acc::widen(ld16u<NTL>((const uint8_t*)t.shard[q] + wg_byte + lane_byte), f);
-            },
-            k, g, first, first_outer, acc);
-        st16<NTS>((u32x4*)(out + head) + v, Acc::narrow(acc));
-      }
+      if (v < nvec)
+        fold_vector<Acc, K, NTL, NTS, PF>(t, k, g, first, first_outer, wg_byte, lane_byte, (u32x4*)(out + head) + v);
     }
 
     // head and tail, by the first tile of the output
@@ -1132,6 +1166,23 @@ __global__ __launch_bounds__(T) void k_reduce_kway(KwayArgs t, int k, int g, int
       out[i] = Acc::narrow1(acc1[0]);
     }
   }
+}
+
+// The same fold for the usual case -- every output, every shard and every
+// element offset 16-byte aligned, n a whole number of vectors: one-wave
+// workgroups on a 2-D grid (y = output, x = 1 KiB tile), nothing decoded by
+// division and nothing peeled.
+template <class Acc, int K, bool NTL, bool NTS, int PF>
+__global__ __launch_bounds__(kRowThreads) void k_fold_rows(KwayArgs t, int k, int g, int first0, size_t nvec) {
+  typedef typename Acc::op::elem elem;
+  const int j = (int)blockIdx.y;
+  const size_t tile_vec = (size_t)blockIdx.x * kRowThreads;
+  if (tile_vec + threadIdx.x >= nvec) return;
+  const int first = g >= k ? (first0 + j) % k : (j % g + 1) % g;
+  const int first_outer = g >= k ? 0 : (j / g + 1) % (k / g);
+  const size_t wg_byte = t.eoff[j] * sizeof(elem) + tile_vec * 16;
+  fold_vector<Acc, K, NTL, NTS, PF>(t, k, g, first, first_outer, wg_byte, threadIdx.x * 16u,
+                                    (u32x4*)t.out[j] + tile_vec + threadIdx.x);
 }
 
 }  // namespace pccl_kernels

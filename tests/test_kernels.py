@@ -480,6 +480,53 @@ def _fold_want(shards, dtype, order, first):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("fold_rows", [1, 0])
+def test_lean_and_general_fold_kernels_agree(target, dtype, fold_rows):
+    """Aligned ring-order folds over up to 16 shards of streams from HBM go to the
+    lean kernel on a 2-D grid (fold_rows = 1, the default; forced at test sizes by
+    the one-wave and non-temporal settings), everything else to the general
+    kernel: both must give the oracle's bits, flat and as whole reduce_scatters."""
+    import torch
+    from pccl import kernels
+    lib = target.native
+    saved = {k: lib.get_tuning(k) for k in ("wg_kway", "nt_load", "nt_store", "lds_pad_kway", "fold_rows")}
+    try:
+        for key, val in (("wg_kway", 64), ("nt_load", 1), ("nt_store", 1), ("fold_rows", fold_rows)):
+            lib.set_tuning(key, val)
+        per_vec = 4 if dtype == O.F32 else 8
+        for k, nvec, pad in ((2, 64, 0), (3, 65, 0), (4, 1, 7168), (5, 200, 0), (8, 129, 8192), (12, 63, 0), (16, 70, 9216), (17, 64, 0)):
+            lib.set_tuning("lds_pad_kway", pad)
+            n = nvec * per_vec
+            shards = make_inputs(k, n, dtype, seed=300 + k)
+            ts = [to_torch(x, dtype, target.device) for x in shards]
+            out = torch.zeros(n, dtype=ts[0].dtype, device=target.device)
+            first = (2 * k // 3) % k
+            print(f"lean fold dtype={dtype} fold_rows={fold_rows} k={k} n={n}", flush=True)
+            lib.reduce_kway(out.data_ptr(), [t.data_ptr() for t in ts], n, CODE[dtype], 0, first, True, target.stream())
+            target.sync()
+            assert_bits_equal(to_numpy(out, dtype), _fold_want(shards, dtype, "ring", first), f"k={k}")
+        lib.set_tuning("lds_pad_kway", 0)
+        for P, B in ((3, 64 * per_vec), (8, 67 * per_vec), (16, 3 * per_vec)):
+            ins = make_inputs(P, P * B, dtype, seed=77 + P)
+            t_in = [to_torch(x, dtype, target.device) for x in ins]
+            t_out = [torch.zeros(B, dtype=t_in[0].dtype, device=target.device) for _ in range(P)]
+            print(f"lean fold reduce_scatter dtype={dtype} fold_rows={fold_rows} P={P} B={B}", flush=True)
+            kernels.reduce_scatter_ranks(t_out, t_in, "ring", "fused")
+            target.sync()
+            want = O.ring_reduce_scatter(ins, dtype)
+            for r in range(P):
+                assert_bits_equal(to_numpy(t_out[r], dtype), want[r], f"P={P} rank {r}")
+            t_io = [t.clone() for t in t_in]                       # in place: output r is block r of input r
+            kernels.reduce_scatter_ranks([t_io[r][r * B:(r + 1) * B] for r in range(P)], t_io, "ring", "fused")
+            target.sync()
+            for r in range(P):
+                assert_bits_equal(to_numpy(t_io[r][r * B:(r + 1) * B].clone(), dtype), want[r], f"in place P={P} rank {r}")
+    finally:
+        for key, val in saved.items():
+            lib.set_tuning(key, val)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("order", ["ring", "halving"])
 def test_one_wave_fold_gives_the_same_bits(target, dtype, order):
     """The fused reduce with one-wave workgroups and paired loads (what streams
