@@ -521,6 +521,18 @@ def test_lean_and_general_fold_kernels_agree(target, dtype, fold_rows):
             target.sync()
             for r in range(P):
                 assert_bits_equal(to_numpy(t_io[r][r * B:(r + 1) * B].clone(), dtype), want[r], f"in place P={P} rank {r}")
+        # a grid beyond the shards of one launch: one fold per node (16 shards), then one per local rank (8)
+        intra, inter, m = 16, 8, 4 * per_vec
+        W = intra * inter
+        ins = make_inputs(W, W * m, dtype, seed=900)
+        t_in = [to_torch(x, dtype, target.device) for x in ins]
+        t_out = [torch.zeros(m, dtype=t_in[0].dtype, device=target.device) for _ in range(W)]
+        print(f"lean fold 2-D {intra}x{inter} dtype={dtype} fold_rows={fold_rows}", flush=True)
+        kernels.reduce_scatter_2d_ranks(t_out, t_in, intra, inter, "ring", "fused")
+        target.sync()
+        want = O.reduce_scatter_2d(ins, intra, inter, dtype, "ring")
+        for w in range(W):
+            assert_bits_equal(to_numpy(t_out[w], dtype), want[w], f"2-D rank {w}")
     finally:
         for key, val in saved.items():
             lib.set_tuning(key, val)
