@@ -525,8 +525,10 @@ struct KwayLaunch {
 // order (butterfly in registers; 8 shards with their loads in pairs): 4 shards
 // bf16 0.81 at 9-10 KiB, fp16 0.815 at 9 KiB, fp32 0.83 at 8 KiB (0.80 without);
 // 8 shards bf16 0.84 and fp16 0.82 at 7 KiB, fp32 0.85 at 11 KiB (0.79); 16 fp32
-// shards 0.80 at 11 KiB (0.76); the kernels for 32 and 64 shards hold 105-182
-// registers per lane, which bounds a CU to 8-16 waves by itself.
+// shards 0.80 at 11 KiB (0.76), 16 bf16 / fp16 shards 0.80 at 14 KiB (0.785 at 11 KiB);
+// 32 fp32 shards 0.83 at 11 KiB, 32 bf16 / fp16 shards 0.80 at 18 KiB (0.775 at 11 KiB);
+// the kernels for 32 and 64 shards hold 105-182 registers per lane, which bounds a
+// CU to 8-16 waves by itself (64 shards: the same at every setting).
 long kway_lds_pad(int k, int g, int dtype, int order, size_t traffic, int threads) {
   if (threads != kRowThreads || !stream_hint(-1, traffic)) return 0;
   if (k <= 2) return 0;
@@ -534,6 +536,8 @@ long kway_lds_pad(int k, int g, int dtype, int order, size_t traffic, int thread
     if (traffic < ((size_t)512 << 20)) return 0;   // not measured below
     if (k == 4) return dtype == PCCL_HIP_F32 ? 8192 : dtype == PCCL_HIP_F16 ? 9216 : 10240;
     if (k == 8) return dtype == PCCL_HIP_F32 ? 11264 : 7168;
+    if (dtype != PCCL_HIP_F32 && k == 16) return 14336;
+    if (dtype != PCCL_HIP_F32 && k == 32) return 18432;
     return 11264;
   }
   const long by_type = dtype == PCCL_HIP_F16 ? -1024 : 0;
