@@ -21,10 +21,10 @@ Workloads:
   cfg1  ring reduce_scatter, P=4, fp32, 16 Mi elements per rank
   cfg2  ring reduce_scatter, P=8, bf16, 256 Mi elements per rank, per-hop
         accumulate with bf16 rounding at every hop
-  cfg2h the cfg2 shape in float16 (the third element type; no BASELINE row)
+  cfg2h the cfg2 shape in float16 (the third element type; not one of the published configurations)
   cfg2d reduce_scatter_2D of the cfg2 data on a grid of 2 nodes x 4 local ranks, ring on
         both levels, as one fused launch (what the reference's harness runs with
-        --library pccl; no BASELINE row)
+        --library pccl; not one of the published configurations)
   cfg3  recursive-halving round at its largest shape: a pair of ranks adding
         512 MiB strided halves (bf16), i.e. round 0 of P=64 with 1 GiB per rank
   cfg3full  the whole recursive-halving reduce_scatter over P=64 resident ranks,
@@ -994,7 +994,7 @@ def cpu_baseline(info):
     job_bytes = 3 * (ranks - 1) * block * (2 if dtype == "bf16" else 4) * ranks
     iters = max(5, min(500, int(10.0 / max(job_bytes / 15e9, 1e-3))))
     head, transport, wall = _cpu_leg(ranks, dtype, block, iters, ["ring"], "0.01" if dtype == "bf16" else "1.0")
-    # BASELINE configuration 1, the one the reference can run on CPUs: P = 4, fp32, blocks of 4 Mi elements
+    # configuration 1 of the published list, the one the reference can run on CPUs: P = 4, fp32, blocks of 4 Mi elements
     c1_ranks = min(4, ranks if ranks >= 2 else 1)
     c1, c1_transport, c1_wall = _cpu_leg(c1_ranks, "f32", 1 << 22, 20, ["ring", "mpi_block"], "1.0")
     cfg1 = {
