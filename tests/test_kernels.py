@@ -586,6 +586,20 @@ def test_one_wave_fold_gives_the_same_bits(target, dtype, order):
             target.sync()
             for r in range(P):
                 assert_bits_equal(to_numpy(t_out[r], dtype), want2[r], f"2-D {alg} 2x{P // 2} rank {r}")
+        # the two-level ring order issues its loads in pairs across the borders of the groups: group sizes
+        # that are even, odd and larger than the number of groups, blocks of whole vectors and ragged ones
+        for intra, inter, m in (((4, 2, 520), (3, 2, 77), (2, 3, 1024), (5, 3, 9), (8, 8, 131), (3, 5, 64), (7, 1, 33), (1, 6, 40))
+                                if order == "ring" else ()):
+            W = intra * inter
+            ins = make_inputs(W, W * m, dtype, seed=500 + W)
+            t_in = [to_torch(x, dtype, target.device) for x in ins]
+            t_out = [torch.zeros(m, dtype=t_in[0].dtype, device=target.device) for _ in range(W)]
+            print(f"one-wave fold 2-D ring {intra}x{inter} m={m} dtype={dtype}", flush=True)
+            kernels.reduce_scatter_2d_ranks(t_out, t_in, intra, inter, "ring", "fused")
+            target.sync()
+            want2 = O.reduce_scatter_2d(ins, intra, inter, dtype, "ring")
+            for w in range(W):
+                assert_bits_equal(to_numpy(t_out[w], dtype), want2[w], f"2-D ring {intra}x{inter} rank {w}")
     finally:
         for k, v in saved.items():
             lib.set_tuning(k, v)
