@@ -19,11 +19,16 @@ DEV = "cuda:0"
 MiB = 1 << 20
 
 
+def _torch_dtype(dtype):
+    import torch
+    return {O.F32: torch.float32, O.BF16: torch.bfloat16, O.F16: torch.float16}[dtype]
+
+
 def _gen(n, dtype, seed, std=1.0, kind="normal"):
     import torch
     g = torch.Generator(device=DEV)
     g.manual_seed(seed)
-    td = torch.float32 if dtype == O.F32 else torch.bfloat16
+    td = _torch_dtype(dtype)
     out = torch.empty(n, dtype=td, device=DEV)
     chunk = 1 << 26
     for i in range(0, n, chunk):
@@ -273,7 +278,8 @@ def test_indexing_beyond_4gib():
 
 @pytest.mark.parametrize("alg,P,dtype", [("ring", 4, O.BF16), ("ring", 16, O.BF16), ("ring", 6, O.F32), ("ring", 16, O.F32),
                                          ("ring", 24, O.F32), ("recursive", 8, O.F32), ("recursive", 16, O.F32),
-                                         ("recursive", 8, O.BF16)])
+                                         ("recursive", 8, O.BF16), ("ring", 8, O.F16), ("recursive", 8, O.F16),
+                                         ("recursive", 32, O.BF16), ("ring", 3, O.F32)])
 def test_fused_reduce_at_streaming_sizes_equals_the_steps(alg, P, dtype):
     """From 288 MiB of traffic on the fused reduce runs with fewer workgroups per
     CU, a number chosen by shard count, element type and order: every such choice
@@ -281,7 +287,7 @@ def test_fused_reduce_at_streaming_sizes_equals_the_steps(alg, P, dtype):
     import torch
     from pccl import kernels
     es = 4 if dtype == O.F32 else 2
-    td = torch.float32 if dtype == O.F32 else torch.bfloat16
+    td = _torch_dtype(dtype)
     B = (1024 * MiB // es // P // P) // 128 * 128 + 8          # about 1 GiB of inputs, blocks not a multiple of a tile
     ins = [_gen(P * B, dtype, 900 + r, kind="int") for r in range(P)]
     total = torch.zeros(P * B, device=DEV)
@@ -306,13 +312,14 @@ def test_fused_reduce_at_streaming_sizes_equals_the_steps(alg, P, dtype):
     _check_rs_windows(outs["fused"], ins, P, B, dtype, alg)
 
 
-@pytest.mark.parametrize("intra,inter,dtype", [(4, 2, O.F32), (4, 2, O.BF16), (4, 4, O.BF16)])
+@pytest.mark.parametrize("intra,inter,dtype", [(4, 2, O.F32), (4, 2, O.BF16), (4, 4, O.BF16), (4, 2, O.F16), (3, 2, O.F32),
+                                               (16, 8, O.BF16)])
 def test_fused_two_level_reduce_at_streaming_sizes_equals_the_steps(intra, inter, dtype):
     import torch
     from pccl import kernels
     W = intra * inter
     es = 4 if dtype == O.F32 else 2
-    td = torch.float32 if dtype == O.F32 else torch.bfloat16
+    td = _torch_dtype(dtype)
     m = (1024 * MiB // es // W // W) // 128 * 128 + 8
     ins = [_gen(W * m, dtype, 700 + r) for r in range(W)]
     outs = {}
