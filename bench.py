@@ -25,6 +25,8 @@ Workloads:
   cfg2d reduce_scatter_2D of the cfg2 data on a grid of 2 nodes x 4 local ranks, ring on
         both levels, as one fused launch (what the reference's harness runs with
         --library pccl; not one of the published configurations)
+  cfg2dh the same with recursive halving on both levels (one 8-way butterfly; what the
+        reference's DeepSpeed patch calls for reduce_scatter_tensor)
   cfg3  recursive-halving round at its largest shape: a pair of ranks adding
         512 MiB strided halves (bf16), i.e. round 0 of P=64 with 1 GiB per rank
   cfg3full  the whole recursive-halving reduce_scatter over P=64 resident ranks,
@@ -65,10 +67,10 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
 MiB = 1 << 20
 WARM_MS = 60.0               # least duration of the untimed warm-up before a timed region, see time_steps
 
-WORKLOADS = ["cfg1", "cfg2", "cfg2h", "cfg2d", "cfg3", "cfg3full", "cfg4", "cfg4u", "cfg5"]
+WORKLOADS = ["cfg1", "cfg2", "cfg2h", "cfg2d", "cfg2dh", "cfg3", "cfg3full", "cfg4", "cfg4u", "cfg5"]
 # every (workload, mode) row of the default run besides the headline cfg2/steps
 ALL_ROWS = [("cfg1", "steps"), ("cfg1", "fused"), ("cfg2", "fused"), ("cfg2h", "steps"), ("cfg2h", "fused"), ("cfg2d", "fused"),
-            ("cfg3", "steps"),
+            ("cfg2dh", "fused"), ("cfg3", "steps"),
             ("cfg3full", "steps"), ("cfg3full", "fused"), ("cfg4", "steps"), ("cfg4", "fused"),
             ("cfg4u", "fused"), ("cfg5", "fused"), ("cfg5", "steps")]
 
@@ -236,10 +238,11 @@ def make_ring_rs(P, elems_per_rank, dtype, modes, device, seed=1234, std=1.0):
     return out
 
 
-def make_grid_rs(intra, inter, elems_per_rank, dtype, modes, device, seed=4321, std=1e-2):
+def make_grid_rs(intra, inter, elems_per_rank, dtype, modes, device, seed=4321, std=1e-2, algorithm="ring"):
     """reduce_scatter_2D (pccl/reduce_scatter.py:205-235) over a grid of inter nodes x intra
-    local ranks, ring order on both levels, as ONE fused launch: what the reference's
-    benchmark harness runs with --library pccl."""
+    local ranks, ring order (or recursive halving, use_rh=True) on both levels, as ONE fused
+    launch: what the reference's benchmark harness runs with --library pccl, and with
+    halving what its DeepSpeed patch calls (pccl/patch_deepspeed.py:42-59)."""
     import torch
     from pccl import kernels
     W = intra * inter
@@ -256,6 +259,15 @@ def make_grid_rs(intra, inter, elems_per_rank, dtype, modes, device, seed=4321, 
     outs = _slab(W, m, tdt, device)
 
     def ring_fold(parts, j):
+        if algorithm != "ring":
+            # the XOR butterfly rooted at j: v[m] = parts[j ^ m]; v[m] += v[m + h] for h = K/2 .. 1
+            v = [parts[j ^ q] for q in range(len(parts))]
+            h = len(parts) // 2
+            while h >= 1:
+                for q in range(h):
+                    v[q] = _hop(v[q], v[q + h])
+                h //= 2
+            return v[0]
         acc = parts[(j + 1) % len(parts)]
         for t in range(2, len(parts) + 1):
             acc = _hop(acc, parts[(j + t) % len(parts)])
@@ -280,16 +292,18 @@ def make_grid_rs(intra, inter, elems_per_rank, dtype, modes, device, seed=4321, 
             raise ValueError("the 2-D workload is measured in the fused mode")
 
         def step():
-            kernels.reduce_scatter_2d_ranks(outs, ins, intra, inter, "ring", "fused")
+            kernels.reduce_scatter_2d_ranks(outs, ins, intra, inter, algorithm, "fused")
 
         nbytes = (W * W + W) * m * es
         out[mode] = (step, dict(
             alg_bytes=nbytes, kernel="k_reduce_kway", kernel_bytes=nbytes, kernel_launches=1, launches=1,
-            desc=f"reduce_scatter_2D, {inter} nodes x {intra} local ranks (virtual), ring on both levels, {dtype}, "
+            desc=f"reduce_scatter_2D, {inter} nodes x {intra} local ranks (virtual), "
+                 f"{'ring' if algorithm == 'ring' else 'recursive halving'} on both levels, {dtype}, "
                  f"{total} elements per rank ({total * es / MiB:.0f} MiB), block {m} elements, mode=fused",
             dtype=dtype, P=W, B=m, verify=verify,
-            verify_how="two-level left fold (locals from local+1, then nodes from node+1) recomputed with torch on "
-                       "windows of blocks 0, W/2, W-1"))
+            verify_how=("two-level left fold (locals from local+1, then nodes from node+1)" if algorithm == "ring" else
+                        "XOR butterfly over the locals rooted at local, then over the nodes rooted at node")
+            + " recomputed with torch on windows of blocks 0, W/2, W-1"))
     return out
 
 
@@ -502,7 +516,7 @@ def make_kway(k, n, modes, device, seed=11):
 
 
 def default_mode(name):
-    return "fused" if name in ("cfg2d", "cfg4", "cfg4u", "cfg5") else "steps"
+    return "fused" if name in ("cfg2d", "cfg2dh", "cfg4", "cfg4u", "cfg5") else "steps"
 
 
 def build_workloads(name, modes, scale, device):
@@ -518,6 +532,8 @@ def build_workloads(name, modes, scale, device):
         return make_ring_rs(8, sc(256 * MiB), "f16", modes, device, std=1e-2)
     if name == "cfg2d":
         return make_grid_rs(4, 2, sc(256 * MiB), "bf16", modes, device)
+    if name == "cfg2dh":
+        return make_grid_rs(4, 2, sc(256 * MiB), "bf16", modes, device, algorithm="recursive")
     if name == "cfg3":
         pair = make_rh_pair(sc(256 * MiB), device)
         return {m: pair["steps"] for m in modes}
