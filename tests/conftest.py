@@ -62,7 +62,7 @@ EMUL_SO = os.path.join(ROOT, "tests", "build", "libpccl_hip_cpu.so")
 HOST_CLANG = "/opt/rocm/lib/llvm/bin/clang++"
 
 
-def build_cpu_library(out=EMUL_SO, extra_flags=()):
+def build_cpu_library(out=EMUL_SO, extra_flags=(), opt="-O1"):
     """Compile the UNCHANGED library source for the host with the stand-in
     <hip/hip_runtime.h> of tests/hip_cpu_shim: each launch then runs the kernel
     thread by thread on the CPU.  Used to check indexing and the host-side
@@ -75,7 +75,7 @@ def build_cpu_library(out=EMUL_SO, extra_flags=()):
     if not os.path.exists(HOST_CLANG):
         pytest.skip("host clang++ of the ROCm toolchain not found")
     os.makedirs(os.path.dirname(out), exist_ok=True)
-    cmd = [HOST_CLANG, "-x", "c++", "-std=c++17", "-O1", "-g", "-fPIC", "-shared", *extra_flags,
+    cmd = [HOST_CLANG, "-x", "c++", "-std=c++17", opt, "-g", "-fPIC", "-shared", *extra_flags,
            "-I", os.path.join(ROOT, "tests", "hip_cpu_shim"), "-I", os.path.join(ROOT, "include"),
            "-I", CSRC, "-o", out, srcs[0]]
     subprocess.run(cmd, check=True, capture_output=True)
