@@ -522,10 +522,10 @@ struct KwayLaunch {
 // settings 4x2 bf16 7 KiB (0.815; 0.77 at 8 KiB), 2x4 6 KiB (0.81; 0.69 at 8 KiB),
 // 3x2 7 KiB, 4x4 7 KiB, 8x8 8 KiB, 16x4 9-10 KiB; fp32 2x4 6 KiB (0.83), 4x2 and
 // 4x4 7 KiB (0.84, 0.81), 6x2 8 KiB, 8x8 8-10 KiB; fp16 4x2 and 4x4 6 KiB.  Halving
-// order (butterfly in registers; 8 shards with their loads in pairs): 4 shards
+// order (butterfly in registers; 8 and 16 shards with their loads in pairs): 4 shards
 // bf16 0.81 at 9-10 KiB, fp16 0.815 at 9 KiB, fp32 0.83 at 8 KiB (0.80 without);
 // 8 shards bf16 0.84 and fp16 0.82 at 7 KiB, fp32 0.85 at 11 KiB (0.79); 16 fp32
-// shards 0.80 at 11 KiB (0.76), 16 bf16 / fp16 shards 0.80 at 14 KiB (0.785 at 11 KiB);
+// shards 0.84 at 11 KiB (0.77), 16 bf16 shards 0.81 at 9-11 KiB (0.76), 16 fp16 shards 0.80 at 8 KiB;
 // 32 fp32 shards 0.83 at 11 KiB, 32 bf16 / fp16 shards 0.80 at 18 KiB (0.775 at 11 KiB);
 // the kernels for 32 and 64 shards hold 105-182 registers per lane, which bounds a
 // CU to 8-16 waves by itself (64 shards: the same at every setting).
@@ -536,7 +536,7 @@ long kway_lds_pad(int k, int g, int dtype, int order, size_t traffic, int thread
     if (traffic < ((size_t)512 << 20)) return 0;   // not measured below
     if (k == 4) return dtype == PCCL_HIP_F32 ? 8192 : dtype == PCCL_HIP_F16 ? 9216 : 10240;
     if (k == 8) return dtype == PCCL_HIP_F32 ? 11264 : 7168;
-    if (dtype != PCCL_HIP_F32 && k == 16) return 14336;
+    if (k == 16) return dtype == PCCL_HIP_F32 ? 11264 : dtype == PCCL_HIP_F16 ? 8192 : 9216;
     if (dtype != PCCL_HIP_F32 && k == 32) return 18432;
     return 11264;
   }

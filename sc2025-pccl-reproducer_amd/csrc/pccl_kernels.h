@@ -920,18 +920,20 @@ __device__ __forceinline__ void tree_sum(Load& load, int first, float* out) {
     tree_sum<Acc, K, M, 2 * H, L>(load, first, lo);
     tree_sum<Acc, K, M + H, 2 * H, L>(load, first, hi);
 #if defined(__HIP_DEVICE_COMPILE__)
-    // Eight shards: the two leaves of a pair are loaded together, ahead of their
+    // Eight and sixteen shards: the two leaves of a pair are loaded together, ahead of their
     // add, and the next pair is not loaded before this one is summed (the sum must
     // exist at the second fence: an empty asm takes it as operand): two loads in
     // flight per wave, as in the ring order.  Left alone, the scheduler issues 6 of
     // the 8 loads up front for the 16-bit types and sinks every fp32 load down to
-    // its add (an asm statement); both measured 4-6 % slower on MI355X.  Four
-    // shards measured the same or slower with the fences and stay without.
-    if constexpr (2 * H == K && K == 8) __builtin_amdgcn_sched_barrier(0);
+    // its add (an asm statement); both measured 4-6 % slower on MI355X (sixteen
+    // shards: 2 % slower as subtrees side by side, see tree_vec).  Four shards
+    // measured the same or slower with the fences and stay without; 32 and 64
+    // shards are faster as subtrees side by side.
+    if constexpr (2 * H == K && (K == 8 || K == 16)) __builtin_amdgcn_sched_barrier(0);
 #endif
     Acc::template join_lanes<L>(lo, hi);
 #if defined(__HIP_DEVICE_COMPILE__)
-    if constexpr (2 * H == K && K == 8) {
+    if constexpr (2 * H == K && (K == 8 || K == 16)) {
 #pragma unroll
       for (int l = 0; l < L; ++l) asm volatile("" : "+v"(lo[l]));
       __builtin_amdgcn_sched_barrier(0);
@@ -984,10 +986,10 @@ __device__ __forceinline__ void tree_vec(Load& load, u32x4* out) {
   }
 }
 
-// Subtrees evaluated side by side for a butterfly over K >= 16 operands (measured:
-// 8 for K = 64 and 32, 4 or 8 alike for K = 16; K = 8 is faster depth first).
+// Subtrees evaluated side by side for a butterfly over K >= 32 operands (measured:
+// 8 for K = 64 and 32; K = 8 and 16 are faster depth first with their leaves in pairs).
 template <int K>
-constexpr int tree_group() { return K >= 32 ? 8 : 4; }
+constexpr int tree_group() { return 8; }
 
 // Left fold over `count` operands in cyclic order first, first+1, ...
 // load(q, f) fills the L fp32 lanes of operand q; acc receives the result.
@@ -1071,7 +1073,7 @@ template <class Acc, int K, bool NTL, bool NTS, int PF>
 __device__ __forceinline__ void fold_vector(const KwayArgs& t, int k, int g, int first, int first_outer,
                                             size_t wg_byte, uint32_t lane_byte, u32x4* dst) {
   constexpr int L = Acc::kLanes;
-  if constexpr (K >= 16 && Acc::kPacked) {
+  if constexpr (K >= 32 && Acc::kPacked) {
     constexpr int G = tree_group<K>();
     u32x4 part[G];
     auto group_load = [&](int b, u32x4* x) {
