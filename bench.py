@@ -27,6 +27,7 @@ Workloads:
         --library pccl; not one of the published configurations)
   cfg2dh the same with recursive halving on both levels (one 8-way butterfly; what the
         reference's DeepSpeed patch calls for reduce_scatter_tensor)
+  cfg2ar all_reduce of the cfg2 data: ring reduce_scatter + all_gather, one fused launch each
   cfg3  recursive-halving round at its largest shape: a pair of ranks adding
         512 MiB strided halves (bf16), i.e. round 0 of P=64 with 1 GiB per rank
   cfg3full  the whole recursive-halving reduce_scatter over P=64 resident ranks,
@@ -67,10 +68,10 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
 MiB = 1 << 20
 WARM_MS = 60.0               # least duration of the untimed warm-up before a timed region, see time_steps
 
-WORKLOADS = ["cfg1", "cfg2", "cfg2h", "cfg2d", "cfg2dh", "cfg3", "cfg3full", "cfg4", "cfg4u", "cfg5"]
+WORKLOADS = ["cfg1", "cfg2", "cfg2h", "cfg2d", "cfg2dh", "cfg2ar", "cfg3", "cfg3full", "cfg4", "cfg4u", "cfg5"]
 # every (workload, mode) row of the default run besides the headline cfg2/steps
 ALL_ROWS = [("cfg1", "steps"), ("cfg1", "fused"), ("cfg2", "fused"), ("cfg2h", "steps"), ("cfg2h", "fused"), ("cfg2d", "fused"),
-            ("cfg2dh", "fused"), ("cfg3", "steps"),
+            ("cfg2dh", "fused"), ("cfg2ar", "fused"), ("cfg3", "steps"),
             ("cfg3full", "steps"), ("cfg3full", "fused"), ("cfg4", "steps"), ("cfg4", "fused"),
             ("cfg4u", "fused"), ("cfg5", "fused"), ("cfg5", "steps")]
 
@@ -235,6 +236,58 @@ def make_ring_rs(P, elems_per_rank, dtype, modes, device, seed=1234, std=1.0):
                  f"({total * es / MiB:.0f} MiB), block {B} elements, mode={_mode_name(m)}",
             dtype=dtype, P=P, B=B, verify=verify,
             verify_how="left fold from rank j+1 recomputed with torch on windows of blocks 0, P/2, P-1"))
+    return out
+
+
+def make_all_reduce(P, elems_per_rank, dtype, modes, device, seed=2468, std=1e-2):
+    """all_reduce = reduce_scatter + all_gather with the ring schedules (pccl/all_reduce.py:21-55,
+    pccl/src/yacl.cpp:146-177), each as one fused launch; the gathered sums land in separate
+    buffers so that every timed call reduces the same inputs."""
+    import torch
+    from pccl import kernels
+    B = elems_per_rank // P
+    total = B * P
+    tdt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dtype]
+    es = 4 if dtype == "f32" else 2
+    ins = _slab(P, total, tdt, device)
+    for r in range(P):
+        if dtype == "f32":
+            _rand_f32(total, seed + r, device, out=ins[r])
+        else:
+            _randn_bf16(total, std, seed + r, device, out=ins[r])
+    blocks = _slab(P, B, tdt, device)
+    sums = _slab(P, total, tdt, device)
+
+    def verify():
+        torch.cuda.synchronize()
+        for j in sorted({0, P // 2, P - 1}):
+            for lo, hi in _windows(B):
+                acc = ins[(j + 1) % P][j * B + lo:j * B + hi]
+                for t in range(2, P + 1):
+                    acc = _hop(acc, ins[(j + t) % P][j * B + lo:j * B + hi])
+                for r in (0, P - 1):
+                    if not _same_bits(sums[r][j * B + lo:j * B + hi], acc):
+                        return False
+        return True
+
+    out = {}
+    for mode in modes:
+        if kernels.mode_code(mode) != kernels.MODE_FUSED:
+            raise ValueError("the all_reduce workload is measured in the fused mode")
+
+        def step():
+            kernels.reduce_scatter_ranks(blocks, ins, "ring", "fused")
+            kernels.all_gather_ranks(sums, blocks, "ring", "fused")
+
+        nbytes = 2 * (P * P + P) * B * es     # the fold reads P*P*B and writes P*B; the placement reads P*B and writes P*P*B
+        out[mode] = (step, dict(
+            alg_bytes=nbytes, kernel="k_fold_rows + k_gather_strips", kernel_bytes=nbytes // 2, kernel_launches=2,
+            launches=2,
+            desc=f"all_reduce = ring reduce_scatter + all_gather, P={P} virtual ranks, {dtype}, {total} elements per rank "
+                 f"({total * es / MiB:.0f} MiB), one fused launch each",
+            dtype=dtype, P=P, B=B, verify=verify,
+            verify_how="every block of the gathered sums of ranks 0 and P-1 against the left fold from rank j+1, "
+                       "recomputed with torch on windows of blocks 0, P/2, P-1"))
     return out
 
 
@@ -516,7 +569,7 @@ def make_kway(k, n, modes, device, seed=11):
 
 
 def default_mode(name):
-    return "fused" if name in ("cfg2d", "cfg2dh", "cfg4", "cfg4u", "cfg5") else "steps"
+    return "fused" if name in ("cfg2d", "cfg2dh", "cfg2ar", "cfg4", "cfg4u", "cfg5") else "steps"
 
 
 def build_workloads(name, modes, scale, device):
@@ -532,6 +585,8 @@ def build_workloads(name, modes, scale, device):
         return make_ring_rs(8, sc(256 * MiB), "f16", modes, device, std=1e-2)
     if name == "cfg2d":
         return make_grid_rs(4, 2, sc(256 * MiB), "bf16", modes, device)
+    if name == "cfg2ar":
+        return make_all_reduce(8, sc(256 * MiB), "bf16", modes, device)
     if name == "cfg2dh":
         return make_grid_rs(4, 2, sc(256 * MiB), "bf16", modes, device, algorithm="recursive")
     if name == "cfg3":
