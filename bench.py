@@ -37,7 +37,7 @@ Workloads:
   cfg5  fused one-pass reduce of 32 fp32 shards of 32 Mi elements
   ceilings  what the device sustains for plain streams of 1 GiB (read-only,
         write-only, copy, add) and for read:write mixes with no data flowing
-        from the loads to the stores (2:1, 8:1, 32:1, 1:16)
+        from the loads to the stores (1:1, 2:1, 8:1, 32:1, 1:16)
   sweep  GB/s against message size, 64 MiB .. 2 GiB per operand
   latency  small messages, 4 KiB .. 1 MiB in bf16: microseconds per call
   placement  the cfg2 shape on six separately allocated groups of buffers in one
@@ -755,7 +755,7 @@ def ceilings(steps, warmup, device):
     # probes are reference points, not bounds: a ratio above 1 says that the library
     # kernel orders its work better than any of the probe's plain shapes.
     mixes = {}
-    for nr, nw, mib in ((2, 1, 1024), (8, 1, 256), (32, 1, 128), (1, 16, 128)):
+    for nr, nw, mib in ((1, 1, 1024), (2, 1, 1024), (8, 1, 256), (32, 1, 128), (1, 16, 128)):
         nb = mib * MiB
         rd = [torch.empty(nb // 4, device=device).normal_() for _ in range(nr)]
         wr = [torch.empty(nb // 4, device=device) for _ in range(nw)]
@@ -766,7 +766,9 @@ def ceilings(steps, warmup, device):
                 v = gbps(lambda: lib.probe_mix(rp, wp, nb, sh, u, st), (nr + nw) * nb)
                 if v > best:
                     best, shape = v, f"shape {sh}, {u} vectors per thread"
-        if nw == 1 and nr == 2:
+        if nw == 1 and nr == 1:
+            mine, kname = gbps(lambda: kernels.copy(wr[0], rd[0]), 2 * nb), "k_copy_segs"
+        elif nw == 1 and nr == 2:
             mine, kname = gbps(lambda: kernels.add(wr[0], rd[0], rd[1]), 3 * nb), "k_add_rows"
         elif nw == 1:
             mine, kname = gbps(lambda: kernels.reduce_kway(wr[0], rd, "ring", 1), (nr + 1) * nb), \
