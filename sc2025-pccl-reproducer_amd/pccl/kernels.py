@@ -331,7 +331,6 @@ def plan_reduce_scatter(outputs: Sequence[torch.Tensor], inputs: Sequence[torch.
                         work: Optional[Sequence[torch.Tensor]] = None) -> CollectivePlan:
     """Validate like reduce_scatter_ranks, then return a callable that replays
     the collective on the same buffers."""
-    import ctypes
     P = len(inputs)
     m = mode_code(mode)
     total = inputs[0].numel()

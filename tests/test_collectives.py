@@ -4,8 +4,7 @@ per-rank API run SPMD (one thread per virtual rank) with both backends."""
 import numpy as np
 import pytest
 
-from helpers import (assert_bits_equal, halving_closed_form, make_inputs, ring_closed_form, to_numpy,
-                     to_torch)
+from helpers import assert_bits_equal, make_inputs, ring_closed_form, to_numpy, to_torch
 from oracle import pccl_oracle as O
 
 DTYPES = [O.F32, O.BF16]

@@ -3,7 +3,6 @@ argument checks of the extension entry points, dispatch precedence.  CPU only;
 where data has to move it goes through the CPU build of the library."""
 import threading
 
-import numpy as np
 import pytest
 
 from oracle import pccl_oracle as O

@@ -1,7 +1,6 @@
 """Randomised shapes on the CPU build: any P, block length, dtype, algorithm,
 mode and operand misalignment must give the oracle's bits."""
 import numpy as np
-import pytest
 from hypothesis import HealthCheck, assume, given, settings, strategies as st
 
 from helpers import assert_bits_equal, make_inputs, to_numpy, to_torch

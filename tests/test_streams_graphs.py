@@ -1,7 +1,6 @@
 """Stream handling: work goes to the caller's current stream, and a whole
 collective (launches only, no allocation, no memset) can be captured in a HIP
 graph and replayed."""
-import numpy as np
 import pytest
 
 from helpers import assert_bits_equal, make_inputs, to_numpy, to_torch

@@ -3,7 +3,6 @@ work buffers are the library's built-in scratch array.  Called through the C ABI
 and compared bit for bit with pccl_hip_reduce_scatter_virtual (per-step mode,
 caller-owned work buffers) and with the oracle, on two calls in a row, the
 second with a smaller input (the scratch keeps the first call's contents)."""
-import numpy as np
 import pytest
 
 from helpers import assert_bits_equal, make_inputs, to_numpy, to_torch
